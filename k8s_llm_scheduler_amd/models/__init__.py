@@ -15,10 +15,10 @@ def _architecture(c: dict) -> str:
 
 def load_config(name_or_path: str):
     """The configuration object of a preset or checkpoint."""
-    from . import putulorn, rupatar
+    from . import nukizen, putulorn, rupatar
     from .config import get_config
 
-    designs = (putulorn, rupatar)
+    designs = (putulorn, rupatar, nukizen)
     for d in designs:
         if name_or_path in d.PRESETS:
             return d.PRESETS[name_or_path]
@@ -37,6 +37,7 @@ def model_class(cfg):
     """The model class of a configuration object."""
     from .config import LlamaConfig
     from .llama import LlamaModel
+    from .nukizen import NukizenConfig, NukizenModel
     from .putulorn import PutulornConfig, PutulornModel
     from .rupatar import RupatarConfig, RupatarModel
 
@@ -44,6 +45,8 @@ def model_class(cfg):
         return PutulornModel
     if isinstance(cfg, RupatarConfig):
         return RupatarModel
+    if isinstance(cfg, NukizenConfig):
+        return NukizenModel
     if isinstance(cfg, LlamaConfig):
         return LlamaModel
     raise TypeError(f"no model class for {type(cfg).__name__}")

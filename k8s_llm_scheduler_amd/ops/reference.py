@@ -64,9 +64,20 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float,
 
 
 def rope_table(head_dim: int, max_pos: int, theta: float, scaling: Optional[dict] = None) -> torch.Tensor:
-    """[max_pos, head_dim] fp32: cos in [:, :D/2], sin in [:, D/2:] (llama3 or linear scaling if given; linear:
-    every frequency divided by ``factor``).  Angles are formed in float64."""
+    """[max_pos, head_dim] fp32: cos in [:, :D/2], sin in [:, D/2:] (llama3, linear or yarn scaling if given; linear:
+    every frequency divided by ``factor``; yarn: the frequencies between the pairs that make ``fast`` and ``slow``
+    turns over ``original`` positions go over linearly from unscaled to divided by ``factor``, and cos and sin are
+    multiplied by 0.1 ln(factor) + 1).  Angles are formed in float64."""
     inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))
+    mag = 1.0
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "yarn":
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        turn = lambda t: head_dim * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(theta))
+        lo = max(math.floor(turn(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(turn(float(scaling["slow"]))), head_dim - 1)
+        ramp = ((torch.arange(head_dim // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        inv = inv / factor * ramp + inv * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
     if scaling and scaling.get("rope_type", scaling.get("type")) == "linear":
         inv = inv / float(scaling["factor"])
     if scaling and scaling.get("rope_type", scaling.get("type")) == "llama3":
@@ -82,7 +93,7 @@ def rope_table(head_dim: int, max_pos: int, theta: float, scaling: Optional[dict
         inv = torch.where(medium, smoothed, inv_l)
     pos = torch.arange(max_pos, dtype=torch.float64)
     f = torch.outer(pos, inv)
-    return torch.cat([f.cos(), f.sin()], dim=-1).float()
+    return (torch.cat([f.cos(), f.sin()], dim=-1) * mag).float()
 
 
 def _rotate(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
@@ -486,7 +497,7 @@ def write_token_stop(s: int, tok: int, tokens, ctx_inc, hist, steps, stop) -> No
 
 
 # ----------------------------------------------------------------------------- fp32 residual stream, gated activations
-ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_TANH, ACT_SILU, ACT_GELU_ERF = 0, 1, 2, 3, 4
+ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_TANH, ACT_SILU, ACT_GELU_ERF, ACT_RELU, ACT_SOFTCAP = 0, 1, 2, 3, 4, 5, 6
 
 
 def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
@@ -494,10 +505,13 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> to
     return table.index_select(0, ids.long()).float() * scale
 
 
-def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps: float, out_dtype, groups: int = 1):
-    """x (fp32, in place) += mult * branch + rowvec; returns x / sqrt(mean(x^2) + eps) * (offset + w) or None, the
-    mean taken over each of ``groups`` equal consecutive parts of a row by itself."""
-    if branch is not None:
+def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps: float, out_dtype, groups: int = 1,
+            branch2=None):
+    """x (fp32, in place) += mult * (branch + branch2) + rowvec; returns x / sqrt(mean(x^2) + eps) * (offset + w) or
+    None, the mean taken over each of ``groups`` equal consecutive parts of a row by itself."""
+    if branch is not None and branch2 is not None:
+        x.add_((branch.float() + branch2.float()) * mult)
+    elif branch is not None:
         x.add_(branch.float() * mult)
     if rowvec is not None:
         x.add_(rowvec.float())
@@ -510,8 +524,11 @@ def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps:
 
 
 def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, row_scale=None, row_map=None) -> torch.Tensor:
-    """Gated kinds take [T, 2F] = [gate | up] and return [T, F]; ACT_TANH / ACT_SILU / ACT_GELU_ERF are elementwise and
-    take a factor per row: logical row i is row ``row_map[i]`` (or i), its input times ``row_scale[i]``."""
+    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_RELU: relu(g) u) take [T, 2F] = [gate | up] and return [T, F];
+    ACT_TANH / ACT_SILU / ACT_GELU_ERF / ACT_SOFTCAP (limit tanh(x / limit)) are elementwise and take a factor per row:
+    logical row i is row ``row_map[i]`` (or i), its input times ``row_scale[i]``."""
+    if kind == ACT_SOFTCAP:
+        return (limit * torch.tanh(x.float() / limit)).to(x.dtype)
     if kind in (ACT_TANH, ACT_SILU, ACT_GELU_ERF):
         f = x.float()
         if row_scale is not None:
@@ -526,6 +543,8 @@ def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, row_
     g, u = x[..., :F].float(), x[..., F:].float()
     if kind == ACT_GELU_TANH:
         y = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g))) * u
+    elif kind == ACT_RELU:
+        y = torch.relu(g) * u
     else:
         if limit > 0:
             g = g.clamp(max=limit)
@@ -707,32 +726,43 @@ def pool_entry(bt_row, b: int, P: int, bs: int) -> int:
 
 
 def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_sin, positions, slot_mapping, vfirst_in,
-                    vfirst_out, lam: float, H: int, G: int, D: int, V: int, dims: int, eps: float, unit: bool) -> None:
-    """Per token: q (first H D columns of qkv, rewritten in place) and k (at koff) get their bias, the rotation of the
-    pairs (2i, 2i + 1), i < dims / 2, by cos_sin[pos] = [cos | sin], and (``unit``) x / sqrt(mean(x^2) + eps) per head;
-    v (at voff) gets its bias and (``vfirst_in``) becomes (1 - lam) v + lam vfirst_in; ``vfirst_out`` receives v in
-    fp32.  k, v go to kcache [slots, G, D] / vcache [slots, G, V] at the tokens' slots (negative: not written); rows
-    with a negative position are skipped."""
+                    vfirst_out, lam: float, H: int, G: int, D: int, V: int, dims: int, eps: float, unit: bool,
+                    half_layout: bool = False, qnw=None, knw=None) -> None:
+    """Per token: q (first H D columns of qkv, rewritten in place) and k (at koff) get their bias, (``qnw`` / ``knw``)
+    the RMS norm over the whole projection (all heads at once) with that weight, the rotation of the pairs
+    (2i, 2i + 1) -- ``half_layout``: (i, i + dims / 2) --, i < dims / 2, by cos_sin[pos] = [cos | sin], and (``unit``)
+    x / sqrt(mean(x^2) + eps) per head; v (at voff) gets its bias and (``vfirst_in``) becomes (1 - lam) v + lam
+    vfirst_in; ``vfirst_out`` receives v in fp32.  k, v go to kcache [slots, G, D] / vcache [slots, G, V] at the tokens'
+    slots (negative: not written); ``kcache`` None: queries only.  Rows with a negative position are skipped."""
     T = qkv.shape[0]
     live = positions >= 0
     half = dims // 2
     cs = cos_sin[positions.long().clamp(min=0)] if dims else None
 
-    def prep(x, bias, n):
+    def prep(x, bias, n, nw):
         x = x.float().view(T, n, D)
         if bias is not None:
             x = x + bias.float().view(n, D)
+        if nw is not None:
+            x = x * torch.rsqrt(x.pow(2).mean((-2, -1), keepdim=True) + eps) * nw.float().view(n, D)
         if dims:
             c, s = cs[:, None, :half], cs[:, None, half:]
-            a, b = x[..., 0:dims:2], x[..., 1:dims:2]
             x = x.clone()
-            x[..., 0:dims:2], x[..., 1:dims:2] = a * c - b * s, b * c + a * s
+            if half_layout:
+                a, b = x[..., :half].clone(), x[..., half:dims].clone()
+                x[..., :half], x[..., half:dims] = a * c - b * s, b * c + a * s
+            else:
+                a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+                x[..., 0:dims:2], x[..., 1:dims:2] = a * c - b * s, b * c + a * s
         if unit:
             x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
         return x
 
-    q = prep(qkv[:, :H * D], qb, H).reshape(T, H * D)
-    k = prep(qkv[:, koff:koff + G * D], kb, G)
+    q = prep(qkv[:, :H * D], qb, H, qnw).reshape(T, H * D)
+    qkv[live, :H * D] = q[live].to(qkv.dtype)
+    if kcache is None:
+        return
+    k = prep(qkv[:, koff:koff + G * D], kb, G, knw)
     v = qkv[:, voff:voff + G * V].float()
     if vb is not None:
         v = v + vb.float()
@@ -740,7 +770,6 @@ def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_s
         v = (1.0 - lam) * v + lam * vfirst_in
     if vfirst_out is not None:
         vfirst_out[live] = v[live]
-    qkv[live, :H * D] = q[live].to(qkv.dtype)
     ok = live & (slot_mapping >= 0)
     kcache[slot_mapping[ok].long()] = k[ok].to(kcache.dtype)
     vcache[slot_mapping[ok].long()] = v[ok].view(-1, G, V).to(vcache.dtype)
@@ -762,10 +791,13 @@ def window_pool(kpool, vpool, kcache, vcache, block_tables, tok_seq, positions, 
 
 
 def window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_seq, positions, H: int, G: int, D: int,
-                     V: int, window: int, P: int, scale: float, sink: bool, bs: int, out_dtype):
-    """Token t at position p attends the cached tokens max(0, p - window + 1) .. p (window <= 0: all) and the pooled
-    blocks b with b P + P - 1 <= p - window, in one softmax (``sink``: one more unit in the denominator); query head h
-    uses key / value head h // (H / G).  The result times sigmoid(gate) if given.  [T, H V]."""
+                     V: int, window: int, P: int, scale: float, sink: bool, bs: int, out_dtype, chunk: int = 0,
+                     softcap: float = 0.0, sinks=None, gate_per_head: bool = False):
+    """Token t at position p attends the cached tokens max(0, p - window + 1) .. p (window <= 0: all; ``chunk`` > 0
+    instead: the tokens of its own chunk, p - p % chunk .. p) and the pooled blocks b with b P + P - 1 <= p - window,
+    in one softmax (``sink``: one more term e^sinks[h], or one unit, in the denominator); scores q . k * scale, then
+    (``softcap`` > 0) softcap tanh(score / softcap); query head h uses key / value head h // (H / G).  The result times
+    sigmoid(gate) if given ([T, H V], or [T, H] with ``gate_per_head``).  [T, H V]."""
     T = q.shape[0]
     out = torch.zeros(T, H, V)
     qf = q.float().reshape(T, -1)[:, :H * D].view(T, H, D)
@@ -775,6 +807,8 @@ def window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_se
         if p < 0:
             continue
         lo = 0 if window <= 0 else max(0, p - window + 1)
+        if chunk > 0:
+            lo = p - p % chunk
         nb = (p - window + 1) // P if (window > 0 and P > 0 and p - window + 1 >= P) else 0
         bt = block_tables[int(tok_seq[t])].long()
         js = torch.arange(lo, p + 1)
@@ -786,12 +820,17 @@ def window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_se
         for h in range(H):
             g = h // R
             s = (K[:, g] @ qf[t, h]) * scale
-            mx = s.max().clamp(min=0.0) if sink else s.max()
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            s0 = (sinks[h].float() if sinks is not None else torch.zeros(())) if sink else None
+            mx = torch.maximum(s.max(), s0) if sink else s.max()
             e = torch.exp(s - mx)
-            den = e.sum() + (torch.exp(-mx) if sink else 0.0)
+            den = e.sum() + (torch.exp(s0 - mx) if sink else 0.0)
             out[t, h] = (e / den) @ Vv[:, g]
+    if gate is not None and gate_per_head:
+        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
     out = out.reshape(T, H * V)
-    if gate is not None:
+    if gate is not None and not gate_per_head:
         out = out * torch.sigmoid(gate.float())
     return out.to(out_dtype)
 
@@ -860,4 +899,128 @@ def gated_scan(proj, kind: int, cols: dict, fbias, ibias, lower, normw, state, c
         y = (out * normw.float().view(1, 1, V)).reshape(T, H * V)
     else:
         y = out.reshape(T, H * V) * normw.float() * torch.sigmoid(pf[:, cols["g"]:cols["g"] + H * V])
+    return y.to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- short convolutions, delta rule, RG-LRU
+CONV_NONE, CONV_SILU = 0, 1
+
+
+def short_conv(x, w, state, cu_q, seq_slots, positions, in_bias, out_bias, act: int, unit_cols: int, unit_dim: int,
+               scale_cols: int, scale: float, unit_eps: float):
+    """Causal convolution over time per channel, over a varlen batch.  ``x`` [T, C] (any row stride), ``w`` [C, taps]
+    (the last tap is the current token's), inputs x + in_bias, zeros before position 0; the taps - 1 inputs before a
+    portion come from ``state`` [slots, taps - 1, C] fp32, which then receives the portion's last ones.  Then out_bias,
+    the activation, and for the first ``unit_cols`` channels, in groups of ``unit_dim``: v / sqrt(sum(v^2) + unit_eps);
+    the first ``scale_cols`` channels times ``scale``.  Returns fp32 [T, C]."""
+    T, C = x.shape
+    n = w.shape[1]
+    wf = w.float()
+    out = torch.zeros(T, C)
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        slot, p0 = int(seq_slots[s]), int(positions[a])
+        xin = x[a:b].float()
+        if in_bias is not None:
+            xin = xin + in_bias.float()
+        hist = state[slot].clone() if n > 1 else torch.zeros(0, C)
+        for r in range(n - 1):
+            if p0 - (n - 1) + r < 0:
+                hist[r] = 0.0
+        full = torch.cat([hist, xin])
+        y = torch.zeros(b - a, C)
+        for j in range(n):
+            y += wf[:, j] * full[j:j + b - a]
+        out[a:b] = y
+        if n > 1:
+            state[slot] = full[-(n - 1):]
+    if out_bias is not None:
+        out = out + out_bias.float()
+    if act == CONV_SILU:
+        out = out * torch.sigmoid(out)
+    if unit_cols:
+        u = out[:, :unit_cols].reshape(T, unit_cols // unit_dim, unit_dim)
+        out[:, :unit_cols] = (u * torch.rsqrt(u.pow(2).sum(-1, keepdim=True) + unit_eps)).reshape(T, unit_cols)
+    if scale_cols:
+        out[:, :scale_cols] *= scale
+    return out
+
+
+def delta_scan(qkv, proj, cols: dict, neg_a, dt_bias, normw, state, cu_q, seq_slots, positions, H: int, G: int, D: int,
+               V: int, eps: float, out_dtype):
+    """Gated delta rule.  ``qkv`` fp32 [T, G D | G D | H V] (prepared queries, keys, values), ``proj`` fp32 with the
+    columns b (H), a (H) and g (H V) at ``cols``; per head h (queries / keys of head h // (H / G)):
+    decay = exp(neg_a[h] softplus(a + dt_bias[h])), beta = sigmoid(b), S <- decay S, u = beta (v - S^T k),
+    S <- S + k u^T, o = S^T q; y = o / rms(o) * normw [V] * silu(g).  ``state`` [slots, H, D V] fp32."""
+    T = qkv.shape[0]
+    q = qkv[:, :G * D].float().view(T, G, D)
+    k = qkv[:, G * D:2 * G * D].float().view(T, G, D)
+    v = qkv[:, 2 * G * D:2 * G * D + H * V].float().view(T, H, V)
+    pf = proj.float()
+    beta = torch.sigmoid(pf[:, cols["b"]:cols["b"] + H])
+    decay = torch.exp(neg_a.float() * torch.nn.functional.softplus(pf[:, cols["a"]:cols["a"] + H] + dt_bias.float()))
+    gate = pf[:, cols["g"]:cols["g"] + H * V]
+    out = torch.zeros(T, H, V)
+    R = H // G
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        slot = int(seq_slots[s])
+        S = torch.zeros(H, D, V) if int(positions[a]) == 0 else state[slot].view(H, D, V).clone()
+        for t in range(a, b):
+            kk = k[t].repeat_interleave(R, 0)                              # [H, D]
+            qq = q[t].repeat_interleave(R, 0)
+            S = decay[t].view(H, 1, 1) * S
+            u = beta[t].view(H, 1) * (v[t] - torch.einsum("hdv,hd->hv", S, kk))
+            S = S + kk.unsqueeze(2) * u.unsqueeze(1)
+            out[t] = torch.einsum("hdv,hd->hv", S, qq)
+        state[slot] = S.reshape(H, D * V)
+    y = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * normw.float()
+    y = y.reshape(T, H * V) * gate * torch.sigmoid(gate)
+    return y.to(out_dtype)
+
+
+def rglru_scan(u, gates, gate_bias, decay_rate, proj, ycol: int, ybias, state, cu_q, seq_slots, positions, C: int,
+               blocks: int, out_dtype):
+    """Real-gated linear recurrent unit per channel.  ``u`` fp32 [T, C]; ``gates`` fp32 [T, blocks, 2 C / blocks]: per
+    block the logits of the recurrence gate then of the input gate, ``gate_bias`` [blocks, 2 C / blocks] added;
+    r, i = sigmoid of them; a = exp(decay_rate r) (``decay_rate`` [C] <= 0), S <- a S + sqrt(1 - a^2) i u;
+    out = S gelu_tanh(proj[:, ycol + c] + ybias).  ``state`` [slots, C] fp32."""
+    T = u.shape[0]
+    bw = C // blocks
+    z = gates.float().view(T, blocks, 2 * bw) + gate_bias.float().view(blocks, 2 * bw)
+    r = torch.sigmoid(z[..., :bw]).reshape(T, C)
+    i = torch.sigmoid(z[..., bw:]).reshape(T, C)
+    la = decay_rate.float() * r
+    a = torch.exp(la)
+    w = torch.sqrt(-torch.expm1(2.0 * la)) * i * u.float()
+    out = torch.zeros(T, C)
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        lo, hi = cu[s], cu[s + 1]
+        if hi <= lo or int(positions[lo]) < 0:
+            continue
+        slot = int(seq_slots[s])
+        S = torch.zeros(C) if int(positions[lo]) == 0 else state[slot].clone()
+        for t in range(lo, hi):
+            S = a[t] * S + w[t]
+            out[t] = S
+        state[slot] = S
+    g = proj[:, ycol:ycol + C].float() + ybias.float()
+    y = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+    return (out * y).to(out_dtype)
+
+
+def norm_mix(a, wa, b, wb, eps: float, ca: float, cb: float, out_dtype):
+    """ca * a / rms(a) * wa + cb * b / rms(b) * wb  (rows; ``b`` may be None)."""
+    af = a.float()
+    y = ca * af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps) * wa.float()
+    if b is not None:
+        bf = b.float()
+        y = y + cb * bf * torch.rsqrt(bf.pow(2).mean(-1, keepdim=True) + eps) * wb.float()
     return y.to(out_dtype)

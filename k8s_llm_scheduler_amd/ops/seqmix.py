@@ -1,7 +1,7 @@
 """Ops of models with an fp32 residual stream, recurrent / windowed- or latent-attention mixers and mixtures of experts.
 
 Same dispatch rule as the rest of :mod:`..ops`: CUDA (= HIP) tensors always run the gfx950 kernels
-(``stream32.hip``, ``mixers.hip``, ``window_attn.hip``, ``gated_scan.hip``, ``moe.hip``) and raise when the extension is missing; CPU tensors run the fp32
+(``stream32.hip``, ``mixers.hip``, ``window_attn.hip``, ``gated_scan.hip``, ``delta_scan.hip``, ``moe.hip``) and raise when the extension is missing; CPU tensors run the fp32
 reference in :mod:`.reference` (the CPU test-suite).  Every op takes bf16 or true-fp32 activations / weights (the
 ``f32`` flag of the kernels); what a design computes in fp32 regardless (residual sum, recurrent state, decays, router,
 attention scores) is fp32 in both.
@@ -15,7 +15,8 @@ from typing import Optional
 import torch
 
 from . import reference as ref
-from .reference import ACT_GELU_ERF, ACT_GELU_TANH, ACT_SILU, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
+from .reference import ACT_GELU_ERF, ACT_GELU_TANH, ACT_RELU, ACT_SILU, ACT_SOFTCAP, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
+from .reference import CONV_NONE, CONV_SILU  # noqa: F401
 from .reference import SCAN_HGRN2, SCAN_MLSTM  # noqa: F401
 
 BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
@@ -67,8 +68,9 @@ def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> to
 
 def resnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, *, branch: Optional[torch.Tensor] = None,
             mult: float = 1.0, rowvec: Optional[torch.Tensor] = None, offset: float = 0.0,
-            out_dtype=BF16, groups: int = 1) -> Optional[torch.Tensor]:
-    """``x`` (fp32 [T, W], updated in place) += mult * branch + rowvec; returns rms-norm(x) * (offset + w) in
+            out_dtype=BF16, groups: int = 1, branch2: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``x`` (fp32 [T, W], updated in place) += mult * (branch + branch2) + rowvec (two sublayers that read one norm
+    leave two branches); returns rms-norm(x) * (offset + w) in
     ``out_dtype``, or None when ``w`` is None (add only).  ``groups`` > 1: every one of that many equal consecutive
     parts of a row is divided by its own root mean square."""
     if x.dtype != F32:
@@ -76,24 +78,45 @@ def resnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, *, branch: O
     T, W = x.shape
     if groups < 1 or W % groups:
         raise ValueError(f"resnorm: {groups} groups do not divide the width {W}")
-    if not _gpu(x, w, branch, rowvec):
-        return ref.resnorm(x, branch, mult, rowvec, w, offset, eps, out_dtype, groups)
+    if branch is None and branch2 is not None:
+        branch, branch2 = branch2, None
+    if not _gpu(x, w, branch, rowvec, branch2):
+        return ref.resnorm(x, branch, mult, rowvec, w, offset, eps, out_dtype, groups, branch2)
     out = torch.empty(T, W, dtype=out_dtype, device=x.device) if w is not None else None
     f32 = _f32(out_dtype)
-    for t, n in ((branch, "branch"), (rowvec, "rowvec"), (w, "w")):
+    for t, n in ((branch, "branch"), (branch2, "branch2"), (rowvec, "rowvec"), (w, "w")):
         if t is not None and t.dtype != out_dtype:
             raise TypeError(f"{n}: expected {out_dtype}, got {t.dtype}")
-    _native().resnorm(_p(x), _p(branch), float(mult), _p(rowvec), _p(w), float(offset), float(eps), _p(out), T, W,
-                      int(groups), f32, -1)
+    _native().resnorm(_p(x), _p(branch), _p(branch2), float(mult), _p(rowvec), _p(w), float(offset), float(eps),
+                      _p(out), T, W, int(groups), f32, -1)
+    return out
+
+
+def norm_mix(a: torch.Tensor, wa: torch.Tensor, b: Optional[torch.Tensor], wb: Optional[torch.Tensor], eps: float,
+             ca: float = 1.0, cb: float = 1.0, out_dtype=None) -> torch.Tensor:
+    """ca * rms-norm(a) * wa + cb * rms-norm(b) * wb over rows [T, W] (norms in fp32; ``b`` None: the first term
+    only): the outputs of two mixers that run side by side, each normed, joined."""
+    out_dtype = out_dtype or a.dtype
+    if not _gpu(a, wa, b, wb):
+        return ref.norm_mix(a, wa, b, wb, eps, ca, cb, out_dtype)
+    T, W = a.shape
+    if b is not None and (b.shape != a.shape or b.dtype != a.dtype or wb is None):
+        raise ValueError("norm_mix: the two inputs must agree in shape and dtype")
+    out = torch.empty(T, W, dtype=out_dtype, device=a.device)
+    _native().norm_mix(out.data_ptr(), _p(a), _p(wa, a.dtype, "wa"), _p(b), _p(wb, a.dtype, "wb"), float(eps), float(ca),
+                       float(cb), T, W, _f32(a.dtype), _f32(out_dtype), -1)
     return out
 
 
 def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, *,
         row_scale: Optional[torch.Tensor] = None, row_map: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP): [T, 2F] = [gate | up] -> [T, F]; ACT_TANH / ACT_SILU / ACT_GELU_ERF
-    (exact gelu): elementwise.  Elementwise kinds take an fp32 factor per row, ``row_scale`` [T]: logical row i is row
-    ``row_map[i]`` (a permutation; default i) and its input is multiplied by ``row_scale[i]`` before the function."""
-    gated = kind in (ACT_GELU_TANH, ACT_SWISH_CLAMP)
+    """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_RELU = relu(g) u): [T, 2F] = [gate | up] -> [T, F]; ACT_TANH /
+    ACT_SILU / ACT_GELU_ERF (exact gelu) / ACT_SOFTCAP (limit tanh(x / limit)): elementwise.  Elementwise kinds take an
+    fp32 factor per row, ``row_scale`` [T]: logical row i is row ``row_map[i]`` (a permutation; default i) and its
+    input is multiplied by ``row_scale[i]`` before the function."""
+    gated = kind in (ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_RELU)
+    if kind == ACT_SOFTCAP and not limit > 0:
+        raise ValueError("act: a soft cap needs a positive limit")
     if gated and (row_scale is not None or row_map is not None):
         raise ValueError("act: row factors go with the elementwise kinds")
     if not _gpu(x, row_scale, row_map):
@@ -385,19 +408,25 @@ def window_kv_write(kcache: torch.Tensor, vcache: torch.Tensor, qkv: torch.Tenso
                     cos_sin: Optional[torch.Tensor], positions: torch.Tensor, slot_mapping: torch.Tensor, H: int, G: int,
                     D: int, V: int, dims: int, eps: float, unit: bool = True, *,
                     vfirst_in: Optional[torch.Tensor] = None, vfirst_out: Optional[torch.Tensor] = None,
-                    lam: float = 0.0) -> None:
+                    lam: float = 0.0, half_layout: bool = False, qnw: Optional[torch.Tensor] = None,
+                    knw: Optional[torch.Tensor] = None) -> None:
     """Prepares a projected row [q (H D) | ... k (G D at ``koff``) ... v (G V at ``voff``) ...] of every token: biases,
     rotation of the dimension pairs (2i, 2i + 1), i < dims / 2, by ``cos_sin[pos]`` = [cos | sin] (fp32), unit RMS per
     head of q and k (``unit``), value mixing v <- (1 - lam) v + lam ``vfirst_in`` [T, G V] fp32; the first mixing layer
-    leaves its v in ``vfirst_out``.  q is rewritten in place; k and v go to the paged caches [slots, G, D] / [slots, G, V]."""
+    leaves its v in ``vfirst_out``.  q is rewritten in place; k and v go to the paged caches [slots, G, D] / [slots, G, V].
+    ``half_layout``: the rotation pairs dimension i with i + dims / 2 instead.  ``qnw`` [H D] / ``knw`` [G D]: before the
+    rotation the whole projection (all heads at once) is divided by its root mean square and multiplied by the weight.
+    ``kcache`` None (a layer that attends another layer's cache): only the queries are prepared."""
     dt = qkv.dtype
+    if kcache is None:
+        vcache, G, koff, voff = None, 0, 0, 0
     if qkv.dim() != 2 or qkv.stride(1) != 1:
         raise ValueError("window_kv_write: the projected rows must be contiguous")
     if koff + G * D > qkv.shape[1] or voff + G * V > qkv.shape[1] or H * D > qkv.shape[1]:
         raise ValueError("window_kv_write: part offsets exceed the projected row")
     if not _gpu(kcache, vcache, qkv):
         return ref.window_kv_write(kcache, vcache, qkv, koff, voff, qb, kb, vb, cos_sin, positions, slot_mapping,
-                                   vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit)
+                                   vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit, half_layout, qnw, knw)
     T = qkv.shape[0]
     if cos_sin is not None and (cos_sin.shape[1] != dims or cos_sin.dtype != F32):
         raise ValueError("window_kv_write: the angle table must be fp32 [positions, dims]")
@@ -407,7 +436,8 @@ def window_kv_write(kcache: torch.Tensor, vcache: torch.Tensor, qkv: torch.Tenso
     _native().window_kv_write(_p(kcache, dt, "kcache"), _p(vcache, dt, "vcache"), qkv.data_ptr(), qkv.stride(0), koff,
                               voff, _p(qb, dt, "qb"), _p(kb, dt, "kb"), _p(vb, dt, "vb"), _p(cos_sin),
                               _p(positions, I32), _p(slot_mapping, I32), _p(vfirst_in), _p(vfirst_out), float(lam), T, H,
-                              G, D, V, dims, float(eps), int(bool(unit)), _f32(dt), -1)
+                              G, D, V, dims, float(eps), int(bool(unit)), int(bool(half_layout)), _p(qnw, dt, "qnw"),
+                              _p(knw, dt, "knw"), _f32(dt), -1)
 
 
 def window_pool(kpool: torch.Tensor, vpool: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
@@ -446,12 +476,16 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
                      kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, H: int, window: int, P: int, scale: float,
                      sink: bool, block_size: int, cu_q: Optional[torch.Tensor] = None, max_qlen: int = 0,
-                     max_keys: int = 0) -> torch.Tensor:
+                     max_keys: int = 0, *, chunk: int = 0, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None,
+                     gate_per_head: bool = False) -> torch.Tensor:
     """Grouped-query attention over the paged caches [slots, G, D] / [slots, G, V]: the token at position p sees the
     tokens max(0, p - window + 1) .. p (``window`` <= 0: all) and, with ``P`` > 0, the pooled blocks that lie wholly
     before the window (b P + P - 1 <= p - window), all in one softmax; ``sink``: one more unit in the denominator.
     ``q`` [T, >= H D] (row stride free, the prepared queries first), ``gate`` [T, H V] (row stride free): the result is
-    multiplied by sigmoid(gate).  Returns [T, H V].
+    multiplied by sigmoid(gate); ``gate_per_head``: ``gate`` is [T, H], one number per head.  Returns [T, H V].
+    ``chunk`` > 0 (instead of a window): positions are cut into chunks of that many, counted from 0, and a token sees
+    the tokens of its own chunk up to itself.  ``softcap`` > 0: scores become softcap tanh(score / softcap).  ``sinks``
+    [H] fp32 (with ``sink``): the extra term of head h is e^sinks[h] instead of 1.
     ``cu_q`` / ``max_qlen`` (the sequences' query offsets and longest portion): bf16 portions of prompts whose sizes
     fit run on the matrix cores, tiles of consecutive tokens sharing the staged keys; anything else (fp32, single
     tokens, other sizes) on the plain-FMA kernel, which splits the keys of few tokens over several workgroups
@@ -459,11 +493,15 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
     G, D, V = kcache.shape[1], kcache.shape[2], vcache.shape[2]
     if H % G:
         raise ValueError(f"window_attention: {H} query heads over {G} key heads")
+    if chunk > 0 and window > 0:
+        raise ValueError("window_attention: a window or chunks, not both")
     if window <= 0:
         P = 0
+    if sinks is not None and (not sink or sinks.dtype != F32 or sinks.numel() != H):
+        raise ValueError("window_attention: sinks are fp32 [H] and go with sink=True")
     if not _gpu(q, kcache, vcache):
         return ref.window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_seq, positions, H, G, D, V,
-                                    window, P, scale, sink, block_size, q.dtype)
+                                    window, P, scale, sink, block_size, q.dtype, chunk, softcap, sinks, gate_per_head)
     T = q.shape[0]
     dt = q.dtype
     if q.stride(1) != 1 or (gate is not None and (gate.stride(1) != 1 or gate.dtype != dt)):
@@ -477,9 +515,11 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
                                   _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"), _p(vpool, F32, "vpool"),
                                   _p(block_tables, I32, "block_tables"), block_tables.shape[1], _p(cu_q, I32, "cu_q"),
                                   _p(positions, I32), cu_q.shape[0] - 1, int(max_qlen), H, G, D, V, int(window), int(P),
-                                  float(scale), int(bool(sink)), block_size, -1)
+                                  float(scale), int(bool(sink)), block_size, int(chunk), float(softcap), _p(sinks),
+                                  int(bool(gate_per_head)), -1)
         return out
-    ns = window_splits(T, G, window, P, max_keys or block_tables.shape[1] * block_size, nat.window_tile_rows(H, G, D, V))
+    ns = window_splits(T, G, window if chunk <= 0 else chunk, P, max_keys or block_tables.shape[1] * block_size,
+                       nat.window_tile_rows(H, G, D, V))
     pacc = pml = None
     if ns > 1:
         pacc = torch.empty(T * H * ns * V, dtype=F32, device=q.device)
@@ -489,7 +529,8 @@ def window_attention(q: torch.Tensor, gate: Optional[torch.Tensor], kcache: torc
                          _p(kcache, dt, "kcache"), _p(vcache, dt, "vcache"), _p(kpool, F32, "kpool"),
                          _p(vpool, F32, "vpool"), _p(block_tables, I32, "block_tables"), block_tables.shape[1],
                          _p(tok_seq, I32), _p(positions, I32), T, H, G, D, V, int(window), int(P), float(scale),
-                         int(bool(sink)), block_size, ns, _f32(dt), -1)
+                         int(bool(sink)), block_size, ns, int(chunk), float(softcap), _p(sinks), int(bool(gate_per_head)),
+                         _f32(dt), -1)
     return out
 
 
@@ -545,4 +586,107 @@ def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, s
                          _p(fbias, out_dtype, "fbias"), _p(ibias, out_dtype, "ibias"), _p(lower, out_dtype, "lower"),
                          _p(normw, out_dtype, "normw"), _p(state), _p(cu_q, I32), _p(seq_slots, I32),
                          _p(positions, I32), nseq, H, D, V, float(eps), float(cap), _f32(out_dtype), T, Lc, _p(ws), -1)
+    return out
+
+
+# ----------------------------------------------------------------------------- short convolutions, delta rule, RG-LRU
+CONV_MAX_TAPS = 16
+
+
+def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, tok_seq: torch.Tensor,
+               seq_slots: torch.Tensor, positions: torch.Tensor, *, in_bias: Optional[torch.Tensor] = None,
+               out_bias: Optional[torch.Tensor] = None, act: int = CONV_NONE, unit_cols: int = 0, unit_dim: int = 0,
+               scale_cols: int = 0, scale: float = 1.0, unit_eps: float = 1e-6) -> torch.Tensor:
+    """Causal convolution over time per channel over a varlen batch, in fp32.  ``x`` fp32 [T, C] (row stride free),
+    ``w`` fp32 [C, taps] (the last tap is the current token's); inputs are x + in_bias, zeros before position 0; the
+    taps - 1 inputs before a portion come from ``state`` [slots, taps - 1, C] fp32, which then receives the portion's
+    last inputs (a portion at position 0 starts from zeros).  Then out_bias, the activation (CONV_SILU), and, for the
+    first ``unit_cols`` channels in groups of ``unit_dim``, v / sqrt(sum(v^2) + unit_eps); the first ``scale_cols``
+    channels times ``scale``.  Returns fp32 [T, C]."""
+    T, C = x.shape
+    taps = w.shape[1]
+    if x.dtype != F32 or w.dtype != F32 or state.dtype != F32 or x.stride(1) != 1:
+        raise TypeError("short_conv: inputs, taps and state are fp32 with contiguous rows")
+    if w.shape[0] != C or taps < 1 or taps > CONV_MAX_TAPS or state.shape[1:] != (max(taps - 1, 0), C):
+        raise ValueError("short_conv: taps [C, n] and state [slots, n - 1, C] must fit the input")
+    if unit_cols and (unit_dim <= 0 or unit_cols % unit_dim or unit_cols > C or unit_dim > 256):
+        raise ValueError("short_conv: unit groups must tile the leading channels")
+    if scale_cols > C:
+        raise ValueError("short_conv: scale_cols exceeds the channels")
+    if not _gpu(x, w, state):
+        return ref.short_conv(x, w, state, cu_q, seq_slots, positions, in_bias, out_bias, act, unit_cols, unit_dim,
+                              scale_cols, scale, unit_eps)
+    out = torch.empty(T, C, dtype=F32, device=x.device)
+    _native().short_conv(out.data_ptr(), x.data_ptr(), x.stride(0), _p(w), _p(state), _p(cu_q, I32, "cu_q"),
+                         _p(tok_seq, I32, "tok_seq"), _p(seq_slots, I32, "seq_slots"), _p(positions, I32, "positions"),
+                         _p(in_bias, F32, "in_bias"), _p(out_bias, F32, "out_bias"), int(act), T, C, taps,
+                         cu_q.shape[0] - 1, int(unit_cols), int(unit_dim), int(scale_cols), float(scale),
+                         float(unit_eps), -1)
+    return out
+
+
+def delta_scan_max_dim() -> int:
+    return 256
+
+
+def delta_scan(qkv: torch.Tensor, proj: torch.Tensor, cols: dict, neg_a: torch.Tensor, dt_bias: torch.Tensor,
+               normw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
+               positions: torch.Tensor, H: int, G: int, D: int, V: int, eps: float, out_dtype) -> torch.Tensor:
+    """The gated delta rule with a matrix state per head over a varlen batch.  ``qkv`` fp32 [T, G D | G D | H V]: the
+    prepared queries (unit vectors times D^-1/2), keys (unit vectors) and values; ``proj`` fp32 [T, ld] holds the
+    columns ``cols`` b (H: beta = sigmoid), a (H: decay = exp(neg_a softplus(a + dt_bias))) and g (H V: output gate,
+    silu); ``neg_a`` / ``dt_bias`` / ``normw`` fp32 [H] / [H] / [V].  Per head, with the queries / keys of head
+    h // (H / G): S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q; y = o / rms(o) * normw * silu(g).
+    ``state`` [slots, H, D V] fp32 is updated in place (a portion at position 0 starts from zero).  [T, H V]."""
+    T = qkv.shape[0]
+    for t, n in ((qkv, "qkv"), (proj, "proj"), (state, "state"), (neg_a, "neg_a"), (dt_bias, "dt_bias"),
+                 (normw, "normw")):
+        if t.dtype != F32:
+            raise TypeError(f"delta_scan: {n} is fp32")
+    if H % G or qkv.shape[1] != 2 * G * D + H * V or not qkv.is_contiguous() or proj.stride(1) != 1:
+        raise ValueError("delta_scan: qkv must be contiguous [T, G D | G D | H V]")
+    for key, wd in (("b", H), ("a", H), ("g", H * V)):
+        if cols[key] < 0 or cols[key] + wd > proj.shape[1]:
+            raise ValueError(f"delta_scan: part {key!r} exceeds the projected row")
+    if state.shape[1:] != (H, D * V):
+        raise ValueError("delta_scan: state must be [slots, H, D V]")
+    if not _gpu(qkv, proj, state):
+        return ref.delta_scan(qkv, proj, cols, neg_a, dt_bias, normw, state, cu_q, seq_slots, positions, H, G, D, V, eps,
+                              out_dtype)
+    if max(D, V) > delta_scan_max_dim():
+        raise ValueError(f"delta_scan: head sizes {D} x {V} exceed the kernel's {delta_scan_max_dim()}")
+    out = torch.empty(T, H * V, dtype=out_dtype, device=qkv.device)
+    _native().delta_scan(out.data_ptr(), _p(qkv), _p(proj), proj.stride(0), int(cols["b"]), int(cols["a"]),
+                         int(cols["g"]), _p(neg_a), _p(dt_bias), _p(normw), _p(state), _p(cu_q, I32),
+                         _p(seq_slots, I32), _p(positions, I32), cu_q.shape[0] - 1, H, G, D, V, float(eps),
+                         _f32(out_dtype), -1)
+    return out
+
+
+def rglru_scan(u: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor, decay_rate: torch.Tensor,
+               proj: torch.Tensor, ycol: int, ybias: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+               seq_slots: torch.Tensor, positions: torch.Tensor, blocks: int, out_dtype, max_qlen: int = 0
+               ) -> torch.Tensor:
+    """The real-gated linear recurrent unit per channel over a varlen batch.  ``u`` fp32 [T, C] (the convolved
+    branch); ``gates`` fp32 [T, blocks, 2 C / blocks]: per block the logits of the recurrence gate r, then of the
+    input gate i (``gate_bias`` [blocks, 2 C / blocks] added, sigmoid); a = exp(decay_rate r) with ``decay_rate``
+    [C] <= 0; S <- a S + sqrt(1 - a^2) i u; out = S gelu_tanh(proj[:, ycol + c] + ybias[c]).  ``state`` [slots, C]
+    fp32 is updated in place (a portion at position 0 starts from zero).  ``max_qlen``: the longest portion (long
+    portions are cut into time slices that run side by side and are joined exactly)."""
+    T, C = u.shape
+    for t, n in ((u, "u"), (gates, "gates"), (gate_bias, "gate_bias"), (decay_rate, "decay_rate"), (proj, "proj"),
+                 (ybias, "ybias"), (state, "state")):
+        if t.dtype != F32:
+            raise TypeError(f"rglru_scan: {n} is fp32")
+    if C % blocks or gates.numel() != T * 2 * C or not gates.is_contiguous() or not u.is_contiguous():
+        raise ValueError("rglru_scan: gates must be contiguous [T, blocks, 2 C / blocks]")
+    if ycol < 0 or ycol + C > proj.shape[1] or proj.stride(1) != 1 or state.shape[1:] != (C,):
+        raise ValueError("rglru_scan: the gate branch exceeds the projected row, or state is not [slots, C]")
+    if not _gpu(u, gates, state):
+        return ref.rglru_scan(u, gates, gate_bias, decay_rate, proj, ycol, ybias, state, cu_q, seq_slots, positions, C,
+                              blocks, out_dtype)
+    out = torch.empty(T, C, dtype=out_dtype, device=u.device)
+    _native().rglru_scan(out.data_ptr(), _p(u), _p(gates), _p(gate_bias), _p(decay_rate), _p(proj), proj.stride(0),
+                         int(ycol), _p(ybias), _p(state), _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32),
+                         cu_q.shape[0] - 1, C, blocks, int(max_qlen or T), _f32(out_dtype), -1)
     return out

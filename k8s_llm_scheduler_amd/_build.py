@@ -37,7 +37,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -O3 otherwise forms from ordinary float code.  The older kernel files keep the flags they were validated with: with
 # the option on every file, the two-rank fused GEMV all-reduce check of tests/test_multigpu.py reported a wrong sum.
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-NO_PACKED_FP32_FILES = {"stream32.hip", "mixers.hip", "moe.hip", "window_attn.hip", "gated_scan.hip"}
+NO_PACKED_FP32_FILES = {"stream32.hip", "mixers.hip", "moe.hip", "window_attn.hip", "gated_scan.hip", "delta_scan.hip"}
 # the lean module: kernels of the fp32-stream designs, the sampler, the small shared kernels; the block allocator
 LEAN_KERNELS = NO_PACKED_FP32_FILES | {"sampler.hip", "misc.hip", "norm.hip"}
 LEAN_RUNTIME = {"block_allocator.cpp"}

@@ -114,8 +114,21 @@ int k8s_pgemm4(void* out, float* slab, const void* x, const void* W, int M, int 
                int splits, int group_m, const void* res, int rms, float eps, hipStream_t s);
 int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, int vocab, float scale, int f32,
                    hipStream_t s);
-int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset, float eps,
-                void* out, int T, int W, int groups, int f32, hipStream_t s);
+int k8s_resnorm(float* x, const void* branch, const void* branch2, float mult, const void* rowvec, const void* w,
+                float offset, float eps, void* out, int T, int W, int groups, int f32, hipStream_t s);
+int k8s_norm_mix(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, float ca, float cb,
+                 int T, int W, int in_f32, int out_f32, hipStream_t s);
+int k8s_short_conv(float* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
+                   const int* tok_seq, const int* seq_slots, const int* positions, const float* in_bias,
+                   const float* out_bias, int act, int T, int C, int taps, int nseq, int unit_cols, int unit_dim,
+                   int scale_cols, float scale, float unit_eps, hipStream_t s);
+int k8s_delta_scan(void* out, const float* qkv, const float* proj, long ld, int cb, int ca, int cg, const float* neg_a,
+                   const float* dt_bias, const float* normw, float* state, const int* cu_q, const int* seq_slots,
+                   const int* positions, int nseq, int H, int G, int D, int V, float eps, int f32, hipStream_t s);
+int k8s_rglru_scan(void* out, const float* u, const float* gates, const float* gate_bias, const float* rate,
+                   const float* proj, long ld, int ycol, const float* ybias, float* state, const int* cu_q,
+                   const int* seq_slots, const int* positions, int nseq, int C, int blocks, int max_qlen, int f32,
+                   hipStream_t s);
 int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha, const float* row_scale,
             const int* row_map, int f32, hipStream_t s);
 int k8s_gemm_any(void* C, const void* A, const void* W, int M, int N, int K, long lda, long ldw, long ldc, int batch,
@@ -147,7 +160,8 @@ int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E,
 int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long ld, int koff, int voff, const void* qb,
                         const void* kb, const void* vb, const float* cos_sin, const int* positions,
                         const int* slot_mapping, const float* vfirst_in, float* vfirst_out, float lam, int T, int H, int G,
-                        int D, int V, int dims, float eps, int unit, int f32, hipStream_t s);
+                        int D, int V, int dims, float eps, int unit, int half_layout, const void* qnw, const void* knw,
+                        int f32, hipStream_t s);
 int k8s_window_pool(float* kpool, float* vpool, const void* kcache, const void* vcache, const int* block_tables,
                     int max_blocks, const int* tok_seq, const int* positions, int T, int G, int D, int V, int P, int bs,
                     int f32, hipStream_t s);
@@ -155,13 +169,14 @@ int k8s_window_tile_rows(int H, int G, int D, int V);
 int k8s_window_attention(void* out, float* pacc, float* pml, const void* q, long ldq, const void* gate, long ldg,
                          const void* kcache, const void* vcache, const float* kpool, const float* vpool,
                          const int* block_tables, int max_blocks, const int* tok_seq, const int* positions, int T, int H,
-                         int G, int D, int V, int window, int P, float scale, int sink, int bs, int nsplit, int f32,
-                         hipStream_t s);
+                         int G, int D, int V, int window, int P, float scale, int sink, int bs, int nsplit, int chunk,
+                         float softcap, const float* sinkv, int gate_ph, int f32, hipStream_t s);
 int k8s_window_mfma_ok(int H, int G, int D, int V);
 int k8s_window_attention_mfma(void* out, const void* q, long ldq, const void* gate, long ldg, const void* kcache,
                               const void* vcache, const float* kpool, const float* vpool, const int* block_tables,
                               int max_blocks, const int* cu_q, const int* positions, int nseq, int max_qlen, int H, int G,
-                              int D, int V, int window, int P, float scale, int sink, int bs, hipStream_t s);
+                              int D, int V, int window, int P, float scale, int sink, int bs, int chunk, float softcap,
+                              const float* sinkv, int gate_ph, hipStream_t s);
 int k8s_gated_scan_max_dim();
 long long k8s_gated_scan_record(int kind, int D, int V);
 int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf, int cg,
@@ -434,10 +449,38 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                          int64_t s) {
     check(k8s_embed_rows(P<float>(out), P<int>(ids), P(table), T, W, vocab, scale, f32, S(s)), "embed_rows");
   });
-  m.def("resnorm", [](uintptr_t x, uintptr_t branch, float mult, uintptr_t rowvec, uintptr_t w, float offset, float eps,
-                      uintptr_t out, int T, int W, int groups, int f32, int64_t s) {
-    check(k8s_resnorm(P<float>(x), P(branch), mult, P(rowvec), P(w), offset, eps, P(out), T, W, groups, f32, S(s)),
-          "resnorm");
+  m.def("resnorm", [](uintptr_t x, uintptr_t branch, uintptr_t branch2, float mult, uintptr_t rowvec, uintptr_t w,
+                      float offset, float eps, uintptr_t out, int T, int W, int groups, int f32, int64_t s) {
+    check(k8s_resnorm(P<float>(x), P(branch), P(branch2), mult, P(rowvec), P(w), offset, eps, P(out), T, W, groups, f32,
+                      S(s)), "resnorm");
+  });
+  m.def("norm_mix", [](uintptr_t out, uintptr_t a, uintptr_t wa, uintptr_t b, uintptr_t wb, float eps, float ca,
+                       float cb, int T, int W, int in_f32, int out_f32, int64_t s) {
+    check(k8s_norm_mix(P(out), P(a), P(wa), P(b), P(wb), eps, ca, cb, T, W, in_f32, out_f32, S(s)), "norm_mix");
+  });
+  // short convolutions, the gated delta rule, the real-gated linear recurrent unit (delta_scan.hip)
+  m.def("short_conv", [](uintptr_t out, uintptr_t x, long ldx, uintptr_t w, uintptr_t state, uintptr_t cu_q,
+                         uintptr_t tok_seq, uintptr_t seq_slots, uintptr_t positions, uintptr_t in_bias,
+                         uintptr_t out_bias, int act, int T, int C, int taps, int nseq, int unit_cols, int unit_dim,
+                         int scale_cols, float scale, float unit_eps, int64_t s) {
+    check(k8s_short_conv(P<float>(out), P<float>(x), ldx, P<float>(w), P<float>(state), P<int>(cu_q), P<int>(tok_seq),
+                         P<int>(seq_slots), P<int>(positions), P<float>(in_bias), P<float>(out_bias), act, T, C, taps,
+                         nseq, unit_cols, unit_dim, scale_cols, scale, unit_eps, S(s)), "short_conv");
+  });
+  m.def("delta_scan", [](uintptr_t out, uintptr_t qkv, uintptr_t proj, long ld, int cb, int ca, int cg, uintptr_t neg_a,
+                         uintptr_t dt_bias, uintptr_t normw, uintptr_t state, uintptr_t cu_q, uintptr_t seq_slots,
+                         uintptr_t positions, int nseq, int H, int G, int D, int V, float eps, int f32, int64_t s) {
+    check(k8s_delta_scan(P(out), P<float>(qkv), P<float>(proj), ld, cb, ca, cg, P<float>(neg_a), P<float>(dt_bias),
+                         P<float>(normw), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H,
+                         G, D, V, eps, f32, S(s)), "delta_scan");
+  });
+  m.def("rglru_scan", [](uintptr_t out, uintptr_t u, uintptr_t gates, uintptr_t gate_bias, uintptr_t rate,
+                         uintptr_t proj, long ld, int ycol, uintptr_t ybias, uintptr_t state, uintptr_t cu_q,
+                         uintptr_t seq_slots, uintptr_t positions, int nseq, int C, int blocks, int max_qlen, int f32,
+                         int64_t s) {
+    check(k8s_rglru_scan(P(out), P<float>(u), P<float>(gates), P<float>(gate_bias), P<float>(rate), P<float>(proj), ld,
+                         ycol, P<float>(ybias), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions),
+                         nseq, C, blocks, max_qlen, f32, S(s)), "rglru_scan");
   });
   m.def("act", [](uintptr_t out, uintptr_t x, int T, int F, int kind, float limit, float alpha, uintptr_t row_scale,
                   uintptr_t row_map, int f32, int64_t s) {
@@ -499,10 +542,11 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("window_kv_write", [](uintptr_t kcache, uintptr_t vcache, uintptr_t qkv, long ld, int koff, int voff,
                               uintptr_t qb, uintptr_t kb, uintptr_t vb, uintptr_t cos_sin, uintptr_t positions,
                               uintptr_t slots, uintptr_t vfirst_in, uintptr_t vfirst_out, float lam, int T, int H, int G,
-                              int D, int V, int dims, float eps, int unit, int f32, int64_t s) {
+                              int D, int V, int dims, float eps, int unit, int half_layout, uintptr_t qnw,
+                              uintptr_t knw, int f32, int64_t s) {
     check(k8s_window_kv_write(P(kcache), P(vcache), P(qkv), ld, koff, voff, P(qb), P(kb), P(vb), P<float>(cos_sin),
                               P<int>(positions), P<int>(slots), P<float>(vfirst_in), P<float>(vfirst_out), lam, T, H, G,
-                              D, V, dims, eps, unit, f32, S(s)), "window_kv_write");
+                              D, V, dims, eps, unit, half_layout, P(qnw), P(knw), f32, S(s)), "window_kv_write");
   });
   m.def("window_pool", [](uintptr_t kpool, uintptr_t vpool, uintptr_t kcache, uintptr_t vcache, uintptr_t bt,
                           int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int G, int D, int V, int P_,
@@ -514,21 +558,24 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("window_attention", [](uintptr_t out, uintptr_t pacc, uintptr_t pml, uintptr_t q, long ldq, uintptr_t gate,
                                long ldg, uintptr_t kcache, uintptr_t vcache, uintptr_t kpool, uintptr_t vpool,
                                uintptr_t bt, int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int H, int G,
-                               int D, int V, int window, int P_, float scale, int sink, int bs, int nsplit, int f32,
-                               int64_t s) {
+                               int D, int V, int window, int P_, float scale, int sink, int bs, int nsplit, int chunk,
+                               float softcap, uintptr_t sinkv, int gate_ph, int f32, int64_t s) {
     check(k8s_window_attention(P(out), P<float>(pacc), P<float>(pml), P(q), ldq, P(gate), ldg, P(kcache), P(vcache),
                                P<float>(kpool), P<float>(vpool), P<int>(bt), max_blocks, P<int>(tok_seq),
-                               P<int>(positions), T, H, G, D, V, window, P_, scale, sink, bs, nsplit, f32, S(s)),
+                               P<int>(positions), T, H, G, D, V, window, P_, scale, sink, bs, nsplit, chunk, softcap,
+                               P<float>(sinkv), gate_ph, f32, S(s)),
           "window_attention");
   });
   m.def("window_mfma_ok", [](int H, int G, int D, int V) { return k8s_window_mfma_ok(H, G, D, V) != 0; });
   m.def("window_attention_mfma", [](uintptr_t out, uintptr_t q, long ldq, uintptr_t gate, long ldg, uintptr_t kcache,
                                     uintptr_t vcache, uintptr_t kpool, uintptr_t vpool, uintptr_t bt, int max_blocks,
                                     uintptr_t cu_q, uintptr_t positions, int nseq, int max_qlen, int H, int G, int D,
-                                    int V, int window, int P_, float scale, int sink, int bs, int64_t s) {
+                                    int V, int window, int P_, float scale, int sink, int bs, int chunk, float softcap,
+                                    uintptr_t sinkv, int gate_ph, int64_t s) {
     check(k8s_window_attention_mfma(P(out), P(q), ldq, P(gate), ldg, P(kcache), P(vcache), P<float>(kpool),
                                     P<float>(vpool), P<int>(bt), max_blocks, P<int>(cu_q), P<int>(positions), nseq,
-                                    max_qlen, H, G, D, V, window, P_, scale, sink, bs, S(s)), "window_attention_mfma");
+                                    max_qlen, H, G, D, V, window, P_, scale, sink, bs, chunk, softcap, P<float>(sinkv),
+                                    gate_ph, S(s)), "window_attention_mfma");
   });
   m.def("gated_scan_max_dim", []() { return k8s_gated_scan_max_dim(); });
   m.def("gated_scan_record", [](int kind, int D, int V) { return k8s_gated_scan_record(kind, D, V); });

@@ -1,0 +1,352 @@
+// Recurrent mixers fed by short causal convolutions, over varlen batches with per-slot fp32 state:
+//   * short_conv: a causal convolution over time per channel (taps - 1 earlier inputs of a sequence come from the batch
+//     or, before the portion, from the slot's saved inputs; zeros before position 0), bias, silu, and unit vectors over
+//     groups of channels (the prepared queries / keys of the delta rule);
+//   * delta_scan: the gated delta rule with a matrix state per head, S [D key channels][V value channels]:
+//       S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q;  y = o / rms(o) * normw * silu(gate)
+//     with g = exp(neg_a softplus(a + dt_bias)) and beta = sigmoid(b) per head;
+//   * rglru_scan: the real-gated linear recurrent unit per channel,
+//       r, i = sigmoid(gate logits + bias);  a = exp(rate r);  S <- a S + sqrt(1 - a^2) i u;  out = S gelu_tanh(y + bias).
+// Everything here is fp32 (inputs are fp32 projections); only the outputs take the activation type.  Sequence s owns
+// tokens cu_q[s] .. cu_q[s + 1] - 1 and the records of slot seq_slots[s]; a portion that starts at position 0 starts
+// from zero state, so a reused slot needs no clearing; positions[t] < 0 marks an idle row that touches nothing.
+#include "common.h"
+
+namespace k8sllm {
+
+constexpr int CONV_MAX_TAPS = 16;
+
+// One workgroup per token.  The first unit_cols channels go one wave per group of unit_dim (<= 256) channels, the
+// rest one thread per channel.
+__global__ __launch_bounds__(256) void short_conv_kernel(
+    float* __restrict__ out, const float* __restrict__ x, long ldx, const float* __restrict__ w,
+    const float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ tok_seq,
+    const int* __restrict__ seq_slots, const int* __restrict__ positions, const float* __restrict__ in_bias,
+    const float* __restrict__ out_bias, int act, int C, int taps, int unit_cols, int unit_dim, int scale_cols,
+    float scale, float unit_eps) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  if (pos < 0) return;
+  const int seq = tok_seq[t];
+  const int a0 = cu_q[seq];
+  // state row r holds the input of position p0 - (taps - 1) + r, p0 the portion's first position
+  const float* st = state + (size_t)seq_slots[seq] * (taps - 1) * C;
+  auto value = [&](int ch) -> float {
+    float acc = out_bias != nullptr ? out_bias[ch] : 0.f;
+    const float ib = in_bias != nullptr ? in_bias[ch] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      if (pos - back < 0) continue;
+      const int tt = t - back;
+      const float xv = tt >= a0 ? x[(size_t)tt * ldx + ch] + ib : st[(size_t)(taps - 1 + (tt - a0)) * C + ch];
+      acc = fmaf(w[(size_t)ch * taps + j], xv, acc);
+    }
+    if (act == 1) acc = acc / (1.f + expf(-acc));
+    return acc;
+  };
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
+  float* dst = out + (size_t)t * C;
+  const int ngroups = unit_dim > 0 ? unit_cols / unit_dim : 0;
+  for (int gv = wave; gv < ngroups; gv += nw) {
+    float y[4], ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int d = lane + 64 * n;
+      y[n] = d < unit_dim ? value(gv * unit_dim + d) : 0.f;
+      ss += y[n] * y[n];
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss + unit_eps);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const int d = lane + 64 * n, ch = gv * unit_dim + d;
+      if (d < unit_dim) dst[ch] = y[n] * inv * (ch < scale_cols ? scale : 1.f);
+    }
+  }
+  for (int ch = ngroups * unit_dim + tid; ch < C; ch += blockDim.x) dst[ch] = value(ch) * (ch < scale_cols ? scale : 1.f);
+}
+
+// state[slot of s] <- the last taps - 1 inputs of sequence s after this portion (a portion shorter than that keeps the
+// newest of the old ones).  One thread per (sequence, channel); it reads everything it needs before it writes.
+__global__ void conv_save_kernel(float* __restrict__ state, const float* __restrict__ x, long ldx,
+                                 const int* __restrict__ cu_q, const int* __restrict__ seq_slots,
+                                 const int* __restrict__ positions, const float* __restrict__ in_bias, int C, int taps) {
+  const int s = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  const int a0 = cu_q[s], n = cu_q[s + 1] - a0;
+  if (ch >= C || n <= 0) return;
+  const int p0 = positions[a0];
+  if (p0 < 0) return;
+  float* st = state + (size_t)seq_slots[s] * (taps - 1) * C;
+  const float ib = in_bias != nullptr ? in_bias[ch] : 0.f;
+  float v[CONV_MAX_TAPS - 1];
+#pragma unroll
+  for (int r = 0; r < CONV_MAX_TAPS - 1; ++r) {
+    v[r] = 0.f;
+    if (r < taps - 1) {
+      const int rel = n - (taps - 1) + r;      // token of the portion, or (negative) an input before it
+      if (rel >= 0) v[r] = x[(size_t)(a0 + rel) * ldx + ch] + ib;
+      else if (p0 + rel >= 0) v[r] = st[(size_t)(taps - 1 + rel) * C + ch];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < CONV_MAX_TAPS - 1; ++r)
+    if (r < taps - 1) st[(size_t)r * C + ch] = v[r];
+}
+
+// One workgroup per (sequence, head).  Thread (x, c) owns value column x of the CH key channels [c CH, (c + 1) CH) of
+// S.  Per token every thread forms its channels' part of S^T k and S^T q from the state before the update; the parts
+// meet in LDS (one barrier), then every thread has u for its column and updates its channels, and group c = 0 finishes
+// the output from o = g S_old^T q + (q . k) u, which equals S_new^T q.  The next token's inputs are loaded while the
+// current one is computed; k and q rotate through three LDS rows and the partial sums through two, so one barrier per
+// token orders everything (a second one when the value channels span several waves, for the output's norm).
+// blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest that keeps
+// DX NS within 1024 threads.  qkv rows: [q (G D) | k (G D) | v (H V)].
+template <typename TA, int CH>
+__global__ __launch_bounds__(1024) void delta_scan_kernel(
+    TA* __restrict__ out, const float* __restrict__ qkv, const float* __restrict__ proj, long ld, int cb, int ca, int cg,
+    const float* __restrict__ neg_a, const float* __restrict__ dt_bias, const float* __restrict__ normw,
+    float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ seq_slots,
+    const int* __restrict__ positions, int H, int G, int D, int V, float eps) {
+  constexpr int DMAX = 256;
+  __shared__ __attribute__((aligned(16))) float sk[3][DMAX], sq[3][DMAX];
+  __shared__ float pk[2][1024], pq[2][1024], pqk[2][16];
+  __shared__ float red[4];
+  const int s = blockIdx.x, hd = blockIdx.y;
+  const int a0 = cu_q[s], b0 = cu_q[s + 1];
+  if (b0 <= a0) return;
+  const int p0 = positions[a0];
+  if (p0 < 0) return;
+  const int x = threadIdx.x, c = threadIdx.y, NS = blockDim.y, DX = blockDim.x;
+  const bool onv = x < V, ond = x < D;
+  const int i0 = c * CH;
+  const int gq = hd / (H / G);
+  const long row = 2L * G * D + (long)H * V;
+  float* st = state + ((size_t)seq_slots[s] * H + hd) * ((size_t)D * V);
+  float S[CH];
+#pragma unroll
+  for (int e = 0; e < CH; ++e) S[e] = (onv && i0 + e < D && p0 != 0) ? st[(size_t)(i0 + e) * V + x] : 0.f;
+  if (c == 0)
+    for (int e = x; e < 3 * DMAX; e += DX) (&sk[0][0])[e] = (&sq[0][0])[e] = 0.f;
+  const float na = neg_a[hd], dtb = dt_bias[hd];
+  const float nwx = (c == 0 && onv) ? normw[x] : 0.f;
+  float nq = 0.f, nk = 0.f, nv = 0.f, nb = 0.f, nz = 0.f, ng = 0.f;
+  auto fetch = [&](int t) {
+    if (t >= b0) return;
+    const float* r = qkv + (size_t)t * row;
+    const float* pr = proj + (size_t)t * ld;
+    if (onv) nv = r[2L * G * D + (long)hd * V + x];
+    nb = pr[cb + hd];
+    nz = pr[ca + hd];
+    if (c == 0) {
+      if (ond) {
+        nq = r[(long)gq * D + x];
+        nk = r[(long)G * D + (long)gq * D + x];
+      }
+      if (onv) ng = pr[cg + (long)hd * V + x];
+    }
+  };
+  fetch(a0);
+  lds_barrier();                       // the rows are cleared
+  if (c == 0 && ond) {
+    sk[0][x] = nk;
+    sq[0][x] = nq;
+  }
+  lds_barrier();
+  for (int t = a0; t < b0; ++t) {
+    const int i = t - a0, cur = i % 3, nxt = (i + 1) % 3, pb = i & 1;
+    const float cv = nv, cbeta = nb, cz = nz, cgate = ng;
+    fetch(t + 1);
+    float ak[4] = {0.f, 0.f, 0.f, 0.f}, aq[4] = {0.f, 0.f, 0.f, 0.f}, aqk = 0.f;
+#pragma unroll
+    for (int e0 = 0; e0 < CH; e0 += 4) {
+      const f32x4 k4 = *reinterpret_cast<const f32x4*>(&sk[cur][i0 + e0]);
+      const f32x4 q4 = *reinterpret_cast<const f32x4*>(&sq[cur][i0 + e0]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ak[e] = fmaf(k4[e], S[e0 + e], ak[e]);
+        aq[e] = fmaf(q4[e], S[e0 + e], aq[e]);
+        aqk = fmaf(k4[e], q4[e], aqk);
+      }
+    }
+    pk[pb][c * DX + x] = (ak[0] + ak[1]) + (ak[2] + ak[3]);
+    pq[pb][c * DX + x] = (aq[0] + aq[1]) + (aq[2] + aq[3]);
+    if (x == 0) pqk[pb][c] = aqk;
+    if (c == 0 && ond && t + 1 < b0) {
+      sk[nxt][x] = nk;
+      sq[nxt][x] = nq;
+    }
+    lds_barrier();
+    float kS = 0.f;
+    for (int g = 0; g < NS; ++g) kS += pk[pb][g * DX + x];
+    const float zz = cz + dtb;
+    const float sp = zz > 20.f ? zz : log1pf(expf(zz));
+    const float decay = expf(na * sp);
+    const float beta = 1.f / (1.f + expf(-cbeta));
+    const float u = beta * (cv - decay * kS);
+#pragma unroll
+    for (int e0 = 0; e0 < CH; e0 += 4) {
+      const f32x4 k4 = *reinterpret_cast<const f32x4*>(&sk[cur][i0 + e0]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) S[e0 + e] = fmaf(k4[e], u, decay * S[e0 + e]);
+    }
+    float o = 0.f, ss = 0.f;
+    if (c == 0) {
+      float qS = 0.f, qk = 0.f;
+      for (int g = 0; g < NS; ++g) {
+        qS += pq[pb][g * DX + x];
+        qk += pqk[pb][g];
+      }
+      o = onv ? fmaf(qk, u, decay * qS) : 0.f;
+      ss = wave_sum(o * o);
+      if (DX > 64 && (x & 63) == 0) red[x >> 6] = ss;
+    }
+    if (DX > 64) {                     // the value channels span several waves: one more exchange (uniform branch)
+      lds_barrier();
+      ss = red[0];
+      for (int w = 1; w < DX / 64; ++w) ss += red[w];
+    }
+    if (c == 0 && onv) {
+      const float y = o / sqrtf(ss / (float)V + eps) * nwx * (cgate / (1.f + expf(-cgate)));
+      stf(out, (size_t)t * H * V + (size_t)hd * V + x, y);
+    }
+  }
+  if (onv) {
+#pragma unroll
+    for (int e = 0; e < CH; ++e)
+      if (i0 + e < D) st[(size_t)(i0 + e) * V + x] = S[e];
+  }
+}
+
+// One workgroup per (sequence, 64 channels); blockDim = (64, NT).  A long portion is cut into NT time slices that run
+// side by side: every slice first composes its own tokens into (A, B) with S_out = A S_in + B, the slices' start states
+// follow from the slot's state by walking the earlier slices' pairs, then every slice runs again from its start state
+// and writes outputs.  NT == 1 (decoding, short portions): one pass.
+template <typename TA>
+__global__ __launch_bounds__(1024) void rglru_scan_kernel(
+    TA* __restrict__ out, const float* __restrict__ u, const float* __restrict__ gates,
+    const float* __restrict__ gate_bias, const float* __restrict__ rate, const float* __restrict__ proj, long ld,
+    int ycol, const float* __restrict__ ybias, float* __restrict__ state, const int* __restrict__ cu_q,
+    const int* __restrict__ seq_slots, const int* __restrict__ positions, int C, int blocks) {
+  __shared__ float sA[16][64], sB[16][64];
+  const int s = blockIdx.x;
+  const int a0 = cu_q[s], b0 = cu_q[s + 1];
+  if (b0 <= a0) return;
+  const int p0 = positions[a0];
+  if (p0 < 0) return;
+  const int x = threadIdx.x, j = threadIdx.y, NT = blockDim.y;
+  const int ch = blockIdx.y * 64 + x;
+  const bool ok = ch < C;
+  const int n = b0 - a0, L = (n + NT - 1) / NT;
+  const int t0 = min(b0, a0 + j * L), t1 = min(b0, t0 + L);
+  const int bw = C / blocks;
+  const int chc = ok ? ch : 0;
+  const int gr = (chc / bw) * 2 * bw + (chc % bw);          // this channel's recurrence-gate logit; the input gate's is bw on
+  const float br = gate_bias[gr], bi = gate_bias[gr + bw], rt = rate[chc];
+  auto coef = [&](int t, float& a, float& b) {
+    const float* gt = gates + (size_t)t * 2 * C;
+    const float r = 1.f / (1.f + expf(-(gt[gr] + br)));
+    const float ig = 1.f / (1.f + expf(-(gt[gr + bw] + bi)));
+    const float la = rt * r;
+    a = expf(la);
+    b = sqrtf(-expm1f(2.f * la)) * ig * u[(size_t)t * C + chc];
+  };
+  if (NT > 1) {
+    float A = 1.f, B = 0.f;
+    if (ok) {
+#pragma unroll 4
+      for (int t = t0; t < t1; ++t) {
+        float a, b;
+        coef(t, a, b);
+        B = fmaf(a, B, b);
+        A *= a;
+      }
+    }
+    sA[j][x] = A;
+    sB[j][x] = B;
+    __syncthreads();
+  }
+  float* st = state + (size_t)seq_slots[s] * C;
+  float S = (ok && p0 != 0) ? st[chc] : 0.f;
+  for (int jj = 0; jj < j; ++jj) S = fmaf(sA[jj][x], S, sB[jj][x]);
+  if (!ok) return;
+  const float yb = ybias[ch];
+#pragma unroll 4
+  for (int t = t0; t < t1; ++t) {
+    float a, b;
+    coef(t, a, b);
+    S = fmaf(a, S, b);
+    const float g = proj[(size_t)t * ld + ycol + ch] + yb;
+    const float y = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    stf(out, (size_t)t * C + ch, S * y);
+  }
+  if (j == NT - 1) st[ch] = S;
+}
+
+}  // namespace k8sllm
+
+using namespace k8sllm;
+
+extern "C" int k8s_short_conv(float* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
+                              const int* tok_seq, const int* seq_slots, const int* positions, const float* in_bias,
+                              const float* out_bias, int act, int T, int C, int taps, int nseq, int unit_cols,
+                              int unit_dim, int scale_cols, float scale, float unit_eps, hipStream_t s) {
+  if (T <= 0 || nseq <= 0) return 0;
+  if (C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || act < 0 || act > 1) return -1;
+  if (taps > 1 && state == nullptr) return -1;
+  if (unit_cols < 0 || unit_cols > C || (unit_cols > 0 && (unit_dim <= 0 || unit_dim > 256 || unit_cols % unit_dim)))
+    return -1;
+  short_conv_kernel<<<T, 256, 0, s>>>(out, x, ldx, w, state, cu_q, tok_seq, seq_slots, positions, in_bias, out_bias, act,
+                                      C, taps, unit_cols, unit_dim, scale_cols, scale, unit_eps);
+  if (taps > 1) {
+    const dim3 grid(nseq, (C + 255) / 256);
+    if (grid.y > 65535) return -2;
+    conv_save_kernel<<<grid, 256, 0, s>>>(state, x, ldx, cu_q, seq_slots, positions, in_bias, C, taps);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_delta_scan(void* out, const float* qkv, const float* proj, long ld, int cb, int ca, int cg,
+                              const float* neg_a, const float* dt_bias, const float* normw, float* state,
+                              const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int G, int D,
+                              int V, float eps, int f32, hipStream_t s) {
+  if (nseq <= 0) return 0;
+  if (H <= 0 || H > 65535 || G <= 0 || H % G || D <= 0 || D > 256 || V <= 0 || V > 256) return -1;
+  const int m = D > V ? D : V, DX = (m + 63) / 64 * 64;
+  int ch = 16;
+  while (ch < 64 && DX * ((D + ch - 1) / ch) > 1024) ch *= 2;
+  if (DX * ((D + ch - 1) / ch) > 1024) return -2;
+  const dim3 block(DX, (D + ch - 1) / ch);
+#define K8S_DS(TA, CH)                                                                                              \
+  delta_scan_kernel<TA, CH><<<dim3(nseq, H), block, 0, s>>>((TA*)out, qkv, proj, ld, cb, ca, cg, neg_a, dt_bias,    \
+                                                            normw, state, cu_q, seq_slots, positions, H, G, D, V, eps)
+#define K8S_DS_T(TA)                  \
+  do {                                \
+    if (ch == 16) K8S_DS(TA, 16);     \
+    else if (ch == 32) K8S_DS(TA, 32); \
+    else K8S_DS(TA, 64);              \
+  } while (0)
+  if (f32) K8S_DS_T(float);
+  else K8S_DS_T(bf16_t);
+#undef K8S_DS_T
+#undef K8S_DS
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_rglru_scan(void* out, const float* u, const float* gates, const float* gate_bias, const float* rate,
+                              const float* proj, long ld, int ycol, const float* ybias, float* state, const int* cu_q,
+                              const int* seq_slots, const int* positions, int nseq, int C, int blocks, int max_qlen,
+                              int f32, hipStream_t s) {
+  if (nseq <= 0) return 0;
+  if (C <= 0 || blocks <= 0 || C % blocks || (C + 63) / 64 > 65535) return -1;
+  int nt = (max_qlen + 31) / 32;       // time slices of at least 32 tokens
+  nt = nt < 1 ? 1 : (nt > 16 ? 16 : nt);
+  const dim3 grid(nseq, (C + 63) / 64), block(64, nt);
+  if (f32)
+    rglru_scan_kernel<float><<<grid, block, 0, s>>>((float*)out, u, gates, gate_bias, rate, proj, ld, ycol, ybias, state,
+                                                    cu_q, seq_slots, positions, C, blocks);
+  else
+    rglru_scan_kernel<bf16_t><<<grid, block, 0, s>>>((bf16_t*)out, u, gates, gate_bias, rate, proj, ld, ycol, ybias,
+                                                     state, cu_q, seq_slots, positions, C, blocks);
+  return (int)hipGetLastError();
+}

@@ -17,11 +17,12 @@ __global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict
   for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)t * W + i] = ldf(table, (size_t)id * W + i) * scale;
 }
 
-// x[t] += mult * branch[t] + rowvec (each optional), stored back in fp32; then (w != null)
+// x[t] += mult * (branch[t] + branch2[t]) + rowvec (each optional), stored back in fp32; then (w != null)
 // out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (offset + w), the mean taken over each of `groups` equal consecutive parts
 // of the row by itself.  One workgroup per row; groups > 1: one wave per part.
 template <typename TA>
-__global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, const TA* __restrict__ branch, float mult,
+__global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, const TA* __restrict__ branch,
+                                                      const TA* __restrict__ branch2, float mult,
                                                       const TA* __restrict__ rowvec, const TA* __restrict__ w,
                                                       float offset, float eps, TA* __restrict__ out, int W, int groups) {
   __shared__ float red[16];
@@ -30,7 +31,7 @@ __global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, con
   const bool upd = branch != nullptr || rowvec != nullptr;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float v = x[base + i];
-    if (branch != nullptr) v += mult * ldf(branch, base + i);
+    if (branch != nullptr) v += mult * (ldf(branch, base + i) + (branch2 != nullptr ? ldf(branch2, base + i) : 0.f));
     if (rowvec != nullptr) v += ldf(rowvec, i);
     if (upd) x[base + i] = v;
     ss += v * v;
@@ -59,7 +60,8 @@ __global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, con
 }
 
 // kinds: 0 gelu_tanh(g) * u, 1 g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit)
-// (limit <= 0: no clamp) -- both read [T, 2F] = [gate | up]; 2 tanh, 3 silu, 4 erf-gelu: elementwise on [T, F].
+// (limit <= 0: no clamp), 5 relu(g) * u -- these read [T, 2F] = [gate | up]; 2 tanh, 3 silu, 4 erf-gelu,
+// 6 limit * tanh(x / limit): elementwise on [T, F].
 // Elementwise kinds take a factor per row: logical row i is row row_map[i] (or i) and its input is multiplied by
 // row_scale[i] before the function (experts whose router weight scales their input).
 template <typename TA>
@@ -70,15 +72,20 @@ __global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T
     const size_t t = i / F, c = i - t * F;
     float y;
     size_t o = i;
-    if (kind >= 2) {
+    if (kind >= 2 && kind != 5) {
       if (row_map != nullptr) o = (size_t)row_map[t] * F + c;
       float v = ldf(x, o);
       if (row_scale != nullptr) v *= row_scale[t];
-      y = kind == 2 ? tanhf(v) : kind == 3 ? v / (1.f + expf(-v)) : 0.5f * v * (1.f + erff(v * 0.7071067811865476f));
+      y = kind == 2   ? tanhf(v)
+          : kind == 3 ? v / (1.f + expf(-v))
+          : kind == 4 ? 0.5f * v * (1.f + erff(v * 0.7071067811865476f))
+                      : limit * tanhf(v / limit);
     } else {
       float g = ldf(x, t * 2 * F + c), u = ldf(x, t * 2 * F + F + c);
       if (kind == 0) {
         y = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+      } else if (kind == 5) {
+        y = fmaxf(g, 0.f) * u;
       } else {
         if (limit > 0.f) {
           g = fminf(g, limit);
@@ -88,6 +95,37 @@ __global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T
       }
     }
     stf(out, o, y);
+  }
+}
+
+// out[t] = ca * a[t] / rms(a[t]) * wa + cb * b[t] / rms(b[t]) * wb (b optional): the outputs of two mixers that run side
+// by side, each normed over the row in fp32, joined.  One workgroup per row.
+template <typename TA, typename TO>
+__global__ __launch_bounds__(256) void norm_mix_kernel(TO* __restrict__ out, const TA* __restrict__ a,
+                                                       const TA* __restrict__ wa, const TA* __restrict__ b,
+                                                       const TA* __restrict__ wb, float eps, float ca, float cb, int W) {
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * W;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float va = ldf(a, base + i);
+    sa += va * va;
+    if (b != nullptr) {
+      const float vb = ldf(b, base + i);
+      sb += vb * vb;
+    }
+  }
+  sa = block_sum(sa, red);
+  const float ia = ca / sqrtf(sa / (float)W + eps);
+  float ib = 0.f;
+  if (b != nullptr) {   // uniform branch
+    sb = block_sum(sb, red);
+    ib = cb / sqrtf(sb / (float)W + eps);
+  }
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float y = ldf(a, base + i) * ia * ldf(wa, i);
+    if (b != nullptr) y += ldf(b, base + i) * ib * ldf(wb, i);
+    stf(out, base + i, y);
   }
 }
 
@@ -274,23 +312,43 @@ extern "C" int k8s_embed_rows(float* out, const int* ids, const void* table, int
   return (int)hipGetLastError();
 }
 
-extern "C" int k8s_resnorm(float* x, const void* branch, float mult, const void* rowvec, const void* w, float offset,
-                           float eps, void* out, int T, int W, int groups, int f32, hipStream_t s) {
+extern "C" int k8s_resnorm(float* x, const void* branch, const void* branch2, float mult, const void* rowvec,
+                           const void* w, float offset, float eps, void* out, int T, int W, int groups, int f32,
+                           hipStream_t s) {
   if (T <= 0) return 0;
-  if (W <= 0 || (w != nullptr && out == nullptr) || groups < 1 || W % groups) return -1;
+  if (W <= 0 || (w != nullptr && out == nullptr) || groups < 1 || W % groups || (branch2 != nullptr && branch == nullptr))
+    return -1;
   if (f32)
-    resnorm_kernel<float><<<T, 256, 0, s>>>(x, (const float*)branch, mult, (const float*)rowvec, (const float*)w,
-                                            offset, eps, (float*)out, W, groups);
+    resnorm_kernel<float><<<T, 256, 0, s>>>(x, (const float*)branch, (const float*)branch2, mult, (const float*)rowvec,
+                                            (const float*)w, offset, eps, (float*)out, W, groups);
   else
-    resnorm_kernel<bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)branch, mult, (const bf16_t*)rowvec, (const bf16_t*)w,
-                                             offset, eps, (bf16_t*)out, W, groups);
+    resnorm_kernel<bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)branch, (const bf16_t*)branch2, mult,
+                                             (const bf16_t*)rowvec, (const bf16_t*)w, offset, eps, (bf16_t*)out, W,
+                                             groups);
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_norm_mix(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, float ca,
+                            float cb, int T, int W, int in_f32, int out_f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (W <= 0 || a == nullptr || wa == nullptr || (b != nullptr && wb == nullptr)) return -1;
+#define K8S_NM(TA, TO)                                                                                              \
+  norm_mix_kernel<TA, TO><<<T, 256, 0, s>>>((TO*)out, (const TA*)a, (const TA*)wa, (const TA*)b, (const TA*)wb, eps, \
+                                            ca, cb, W)
+  if (in_f32 && out_f32) K8S_NM(float, float);
+  else if (in_f32) K8S_NM(float, bf16_t);
+  else if (out_f32) K8S_NM(bf16_t, float);
+  else K8S_NM(bf16_t, bf16_t);
+#undef K8S_NM
   return (int)hipGetLastError();
 }
 
 extern "C" int k8s_act(void* out, const void* x, int T, int F, int kind, float limit, float alpha,
                        const float* row_scale, const int* row_map, int f32, hipStream_t s) {
   if (T <= 0 || F <= 0) return 0;
-  if (kind < 0 || kind > 4 || (kind < 2 && (row_scale != nullptr || row_map != nullptr))) return -1;
+  const bool gated = kind < 2 || kind == 5;
+  if (kind < 0 || kind > 6 || (gated && (row_scale != nullptr || row_map != nullptr)) || (kind == 6 && !(limit > 0.f)))
+    return -1;
   const size_t n = (size_t)T * F;
   const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
   if (f32) act_kernel<float><<<blocks, 256, 0, s>>>((float*)out, (const float*)x, T, F, kind, limit, alpha,

@@ -4,8 +4,12 @@
 //     b P .. b P + P - 1, seen when b P + P - 1 <= p - window): the mean of the block's cached keys / values;
 //   * tokens and blocks share one softmax, optionally with a sink (a key of score 0 without a value: one more unit
 //     in the denominator);
-//   * queries and keys are prepared by one kernel per token: bias, interleaved-pair rotation of the first `dims`
-//     dimensions, optional unit RMS per head, value mixing with another layer's values, paged cache write.
+//   * instead of a window the mask can be chunked: positions are cut into chunks of `chunk` counted from 0 and a token
+//     sees the tokens of its own chunk up to itself; scores can be soft-capped (cap tanh(s / cap)); the sink can be a
+//     learned number per head (e^sink in the denominator); the output gate is per element or one number per head;
+//   * queries and keys are prepared by one kernel per token: bias, optional RMS norm over the whole projection with a
+//     weight, rotation of the first `dims` dimensions (interleaved pairs or the half layout), optional unit RMS per
+//     head, value mixing with another layer's values, paged cache write (none for a layer that reads another's cache).
 // Varlen batches as in mixers.hip: positions[t] < 0 marks an idle row that touches nothing.
 #include "common.h"
 
@@ -19,7 +23,8 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 // One workgroup per token, one wave per head vector (H query heads, then G key heads; further passes when there are
-// more vectors than waves).  x = proj + bias; (x[2i], x[2i + 1]) turns by the angle of cos_sin[pos] = [cos(dims / 2) |
+// more vectors than waves).  x = proj + bias; (qnw / knw) x = x / rms(whole q or k projection) * weight;
+// (x[2i], x[2i + 1]) -- half layout: (x[i], x[i + dims / 2]) -- turns by the angle of cos_sin[pos] = [cos(dims / 2) |
 // sin(dims / 2)]; then x / sqrt(mean(x^2) + eps) when `unit`.  Queries are written back in place, keys to
 // kcache[slot][g][D].  Values: v = proj + bias, then (vfirst_in) v = (1 - lam) v + lam vfirst_in[t]; (vfirst_out)
 // vfirst_out[t] = v in fp32; vcache[slot][g][V] = v.
@@ -28,8 +33,10 @@ __global__ __launch_bounds__(256) void window_kv_write_kernel(
     TA* __restrict__ kcache, TA* __restrict__ vcache, TA* __restrict__ qkv, long ld, int koff, int voff,
     const TA* __restrict__ qb, const TA* __restrict__ kb, const TA* __restrict__ vb, const float* __restrict__ cos_sin,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping, const float* __restrict__ vfirst_in,
-    float* __restrict__ vfirst_out, float lam, int H, int G, int D, int V, int dims, float eps, int unit) {
+    float* __restrict__ vfirst_out, float lam, int H, int G, int D, int V, int dims, float eps, int unit,
+    int half_layout, const TA* __restrict__ qnw, const TA* __restrict__ knw) {
   extern __shared__ float xs[];   // [waves][D]
+  __shared__ float red[16];
   const int t = blockIdx.x;
   const int pos = positions[t];
   if (pos < 0) return;
@@ -39,12 +46,35 @@ __global__ __launch_bounds__(256) void window_kv_write_kernel(
   const float* cs = cos_sin + (size_t)pos * dims;
   TA* row = qkv + (size_t)t * ld;
   float* x = xs + (size_t)wave * D;
+  float invq = 1.f, invk = 1.f;
+  if (qnw != nullptr) {           // uniform branches: the norm runs over all heads of the projection at once
+    float ss = 0.f;
+    for (int i = tid; i < H * D; i += blockDim.x) {
+      const float v = ldf(row, i) + (qb != nullptr ? ldf(qb, i) : 0.f);
+      ss += v * v;
+    }
+    invq = 1.0f / sqrtf(block_sum(ss, red) / (float)(H * D) + eps);
+  }
+  if (knw != nullptr && G > 0) {
+    float ss = 0.f;
+    for (int i = tid; i < G * D; i += blockDim.x) {
+      const float v = ldf(row + koff, i) + (kb != nullptr ? ldf(kb, i) : 0.f);
+      ss += v * v;
+    }
+    invk = 1.0f / sqrtf(block_sum(ss, red) / (float)(G * D) + eps);
+  }
   for (int hv = wave; hv < H + G; hv += nw) {
     const bool isq = hv < H;
     const int hd = isq ? hv : hv - H;
     const TA* src = row + (isq ? 0 : koff) + (size_t)hd * D;
     const TA* bias = isq ? qb : kb;
-    for (int d = lane; d < D; d += 64) x[d] = ldf(src, d) + (bias != nullptr ? ldf(bias, (size_t)hd * D + d) : 0.f);
+    const TA* nrm = isq ? qnw : knw;
+    const float inv0 = isq ? invq : invk;
+    for (int d = lane; d < D; d += 64) {
+      float v = ldf(src, d) + (bias != nullptr ? ldf(bias, (size_t)hd * D + d) : 0.f);
+      if (nrm != nullptr) v *= inv0 * ldf(nrm, (size_t)hd * D + d);
+      x[d] = v;
+    }
     wave_lds_sync();
     float ss = 0.f;
     float y[8];   // D <= 512
@@ -54,7 +84,13 @@ __global__ __launch_bounds__(256) void window_kv_write_kernel(
       float v = 0.f;
       if (d < D) {
         v = x[d];
-        if (d < dims) {
+        if (d < dims && half_layout) {
+          const bool first = d < half;
+          const int i = first ? d : d - half;
+          const float c = cs[i], sn = cs[half + i];
+          const float a = x[i], b = x[i + half];
+          v = first ? a * c - b * sn : b * c + a * sn;
+        } else if (d < dims) {
           const int i = d >> 1;
           const float c = cs[i], sn = cs[half + i];
           const float a = x[d & ~1], b = x[d | 1];
@@ -157,7 +193,8 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
                                         const int* __restrict__ block_tables, int max_blocks,
                                         const int* __restrict__ tok_seq, const int* __restrict__ positions, int H, int G,
                                         int D, int V, int window, int P, float scale, int sink, int bs, int ppb, int KB,
-                                        int nsplit) {
+                                        int nsplit, int chunk, float softcap, const float* __restrict__ sinkv,
+                                        int gate_ph) {
   extern __shared__ float smem[];
   const int t = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
   const int R = H / G;
@@ -175,7 +212,7 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
   size_t roff = (size_t)KB * (DP + V) + (size_t)nw * D;
   roff += roff & 1;                            // 8-byte aligned
   long long* rowoff = reinterpret_cast<long long*>(smem + roff);   // [KB] a tile row's cache slot, or -1 - pool entry
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int lo = chunk > 0 ? p - p % chunk : (window > 0 ? max(0, p - window + 1) : 0);
   const int nb = (window > 0 && P > 0 && p - window + 1 >= P) ? (p - window + 1) / P : 0;
   const int nkeys = nb + (p + 1 - lo);
   const int ntiles = (nkeys + KB - 1) / KB;
@@ -190,7 +227,7 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
     float* qq = qs + (size_t)wave * D;
     if (hv)
       for (int d = lane; d < D; d += 64) qq[d] = ldf(q, (size_t)t * ldq + (size_t)hd * D + d);
-    float m = with_sink ? 0.f : -INFINITY, l = with_sink ? 1.f : 0.f, acc[NACC];
+    float m = with_sink ? ((sinkv != nullptr && hv) ? sinkv[hd] : 0.f) : -INFINITY, l = with_sink ? 1.f : 0.f, acc[NACC];
 #pragma unroll
     for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
     for (int tile = tile0; tile < tile1; ++tile) {
@@ -246,6 +283,7 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
           float a = 0.f;
           for (int d = 0; d < D; ++d) a = fmaf(qq[d], kr[d], a);
           sc = a * scale;
+          if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
         }
         const float mn = fmaxf(m, wave_max(sc));
         const float alpha = m == -INFINITY ? 0.f : expf(m - mn);
@@ -270,7 +308,8 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
         const int d = lane + 64 * i;
         if (d < V) {
           float o = acc[i] / l;
-          if (gate != nullptr) o *= 1.f / (1.f + expf(-ldf(gate, (size_t)t * ldg + (size_t)hd * V + d)));
+          if (gate != nullptr)
+            o *= 1.f / (1.f + expf(-ldf(gate, (size_t)t * ldg + (gate_ph ? (size_t)hd : (size_t)hd * V + d))));
           stf(out, (size_t)t * H * V + (size_t)hd * V + d, o);
         }
       }
@@ -293,7 +332,7 @@ __global__ void window_attention_kernel(TA* __restrict__ out, float* __restrict_
 template <typename TA>
 __global__ void window_merge_kernel(TA* __restrict__ out, const float* __restrict__ pacc, const float* __restrict__ pml,
                                     const TA* __restrict__ gate, long ldg, const int* __restrict__ positions, int H,
-                                    int V, int nsplit) {
+                                    int V, int nsplit, int gate_ph) {
   const int t = blockIdx.x, hd = blockIdx.y;
   if (positions[t] < 0) {
     for (int d = threadIdx.x; d < V; d += blockDim.x) stf(out, (size_t)t * H * V + (size_t)hd * V + d, 0.f);
@@ -314,7 +353,8 @@ __global__ void window_merge_kernel(TA* __restrict__ out, const float* __restric
       if (ms != -INFINITY) a += expf(ms - M) * pacc[(rec0 + s) * V + d];
     }
     float o = a / den;
-    if (gate != nullptr) o *= 1.f / (1.f + expf(-ldf(gate, (size_t)t * ldg + (size_t)hd * V + d)));
+    if (gate != nullptr)
+      o *= 1.f / (1.f + expf(-ldf(gate, (size_t)t * ldg + (gate_ph ? (size_t)hd : (size_t)hd * V + d))));
     stf(out, (size_t)t * H * V + (size_t)hd * V + d, o);
   }
 }
@@ -337,7 +377,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache, const float* __restrict__ kpool,
     const float* __restrict__ vpool, const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ positions, int H, int G, int D, int V, int window, int P, float scale, int sink, int bs,
-    int ppb, int R) {
+    int ppb, int R, int chunk, float softcap, const float* __restrict__ sinkv, int gate_ph) {
   extern __shared__ __attribute__((aligned(16))) char smem_w[];
   const int seq = blockIdx.z, g = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 15, g4 = lane >> 4;
@@ -358,7 +398,9 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
   char* klds = smem_w;                                   // [32][D + 8] bf16
   char* vlds = smem_w + 32 * rowk;                       // [32][V + 8] bf16
   const bool win = window > 0;
-  const int lo_min = win ? max(0, p_first - window + 1) : 0;
+  // the first position a token at p sees: its chunk's first, the window's first, or 0 (never decreasing in p)
+  auto lo_of = [&](int p) { return chunk > 0 ? p - p % chunk : (win ? max(0, p - window + 1) : 0); };
+  const int lo_min = lo_of(p_first);
   const int nb_max = (win && P > 0 && p_last - window + 1 >= P) ? (p_last - window + 1) / P : 0;
   const int nkeys = nb_max + (p_last + 1 - lo_min);
   const int nsteps = (nkeys + 31) / 32;
@@ -377,7 +419,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     const bool ok = toff < nval;
     c_tok[cb] = tq0 + toff;
     c_p[cb] = ok ? p_first + toff : -1;
-    c_lo[cb] = win ? max(0, c_p[cb] - window + 1) : 0;
+    c_lo[cb] = ok ? lo_of(c_p[cb]) : 0;
     c_nb[cb] = (ok && win && P > 0 && c_p[cb] - window + 1 >= P) ? (c_p[cb] - window + 1) / P : 0;
     const int hd = g * R + li % R;
 #pragma unroll
@@ -394,13 +436,13 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     }
   }
   const bool w_any = w_pmax >= 0;
-  const int w_lo = (w_any && win) ? max(0, w_pmin - window + 1) : 0;
+  const int w_lo = w_any ? lo_of(w_pmin) : 0;
   const int w_nb = (w_any && win && P > 0 && w_pmax - window + 1 >= P) ? (w_pmax - window + 1) / P : 0;
   f32x4 o[NCB][NVB];
   float m_run[NCB], l_run[NCB];
 #pragma unroll
   for (int cb = 0; cb < NCB; ++cb) {
-    m_run[cb] = sink ? 0.f : -INFINITY;
+    m_run[cb] = sink ? (sinkv != nullptr ? sinkv[g * R + li % R] : 0.f) : -INFINITY;
     l_run[cb] = sink ? 1.f : 0.f;
 #pragma unroll
     for (int n = 0; n < NVB; ++n) o[cb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -518,7 +560,11 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
             const int j = lo_min + (u - nb_max);
             vis = j <= c_p[cb] && j >= c_lo[cb];
           }
-          const float v = vis ? sacc[cb][m][i] * scale : -INFINITY;
+          float v = -INFINITY;
+          if (vis) {
+            v = sacc[cb][m][i] * scale;
+            if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+          }
           sacc[cb][m][i] = v;
           tmax = fmaxf(tmax, v);
         }
@@ -589,7 +635,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
         if (n < nvb) {
           const int d = 16 * n + li;
           float y = o[cb][n][i] * inv;
-          if (gate != nullptr) y *= 1.f / (1.f + expf(-bf2f(gate[(size_t)t * ldg + (size_t)hd * V + d])));
+          if (gate != nullptr)
+            y *= 1.f / (1.f + expf(-bf2f(gate[(size_t)t * ldg + (gate_ph ? (size_t)hd : (size_t)hd * V + d)])));
           out[(size_t)t * H * V + (size_t)hd * V + d] = f2bf(y);
         }
     }
@@ -603,15 +650,19 @@ using namespace k8sllm;
 extern "C" int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long ld, int koff, int voff, const void* qb,
                                    const void* kb, const void* vb, const float* cos_sin, const int* positions,
                                    const int* slot_mapping, const float* vfirst_in, float* vfirst_out, float lam, int T,
-                                   int H, int G, int D, int V, int dims, float eps, int unit, int f32, hipStream_t s) {
+                                   int H, int G, int D, int V, int dims, float eps, int unit, int half_layout,
+                                   const void* qnw, const void* knw, int f32, hipStream_t s) {
   if (T <= 0) return 0;
-  if (H <= 0 || G <= 0 || H % G || D <= 0 || D > 512 || V <= 0 || dims < 0 || dims > D || (dims & 1)) return -1;
+  // G == 0: a layer that attends another layer's cache prepares its queries only
+  if (H <= 0 || G < 0 || (G > 0 && H % G) || D <= 0 || D > 512 || V <= 0 || dims < 0 || dims > D || (dims & 1)) return -1;
+  if (G > 0 && (kcache == nullptr || vcache == nullptr)) return -1;
   if (dims > 0 && cos_sin == nullptr) return -1;
   const size_t lds = (size_t)4 * D * sizeof(float);
 #define K8S_WKW(TA)                                                                                                   \
   window_kv_write_kernel<TA><<<T, 256, lds, s>>>((TA*)kcache, (TA*)vcache, (TA*)qkv, ld, koff, voff, (const TA*)qb,    \
                                                  (const TA*)kb, (const TA*)vb, cos_sin, positions, slot_mapping,      \
-                                                 vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit)
+                                                 vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit, half_layout, \
+                                                 (const TA*)qnw, (const TA*)knw)
   if (f32) K8S_WKW(float);
   else K8S_WKW(bf16_t);
 #undef K8S_WKW
@@ -649,7 +700,8 @@ extern "C" int k8s_window_attention(void* out, float* pacc, float* pml, const vo
                                     long ldg, const void* kcache, const void* vcache, const float* kpool,
                                     const float* vpool, const int* block_tables, int max_blocks, const int* tok_seq,
                                     const int* positions, int T, int H, int G, int D, int V, int window, int P,
-                                    float scale, int sink, int bs, int nsplit, int f32, hipStream_t s) {
+                                    float scale, int sink, int bs, int nsplit, int chunk, float softcap,
+                                    const float* sinkv, int gate_ph, int f32, hipStream_t s) {
   if (T <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || V <= 0 || V > 256 || bs <= 0 || G > 65535) return -1;
   if (window > 0 && P > 0 && (kpool == nullptr || vpool == nullptr)) return -1;
@@ -665,7 +717,8 @@ extern "C" int k8s_window_attention(void* out, float* pacc, float* pml, const vo
 #define K8S_WA(TA, NA, VEC)                                                                                           \
   window_attention_kernel<TA, NA, VEC><<<dim3(T, G, nsplit), nw * 64, lds, s>>>(                                      \
       (TA*)out, pacc, pml, (const TA*)q, ldq, (const TA*)gate, ldg, (const TA*)kcache, (const TA*)vcache, kpool,      \
-      vpool, block_tables, max_blocks, tok_seq, positions, H, G, D, V, window, P, scale, sink, bs, ppb, KB, nsplit)
+      vpool, block_tables, max_blocks, tok_seq, positions, H, G, D, V, window, P, scale, sink, bs, ppb, KB, nsplit,   \
+      chunk, softcap, sinkv, gate_ph)
 #define K8S_WA_V(TA, NA)            \
   do {                              \
     if (vec) K8S_WA(TA, NA, true);  \
@@ -685,10 +738,10 @@ extern "C" int k8s_window_attention(void* out, float* pacc, float* pml, const vo
   if (nsplit > 1) {
     if (f32)
       window_merge_kernel<float><<<dim3(T, H), 64, 0, s>>>((float*)out, pacc, pml, (const float*)gate, ldg, positions, H,
-                                                           V, nsplit);
+                                                           V, nsplit, gate_ph);
     else
       window_merge_kernel<bf16_t><<<dim3(T, H), 64, 0, s>>>((bf16_t*)out, pacc, pml, (const bf16_t*)gate, ldg,
-                                                            positions, H, V, nsplit);
+                                                            positions, H, V, nsplit, gate_ph);
   }
   return (int)hipGetLastError();
 }
@@ -705,7 +758,8 @@ extern "C" int k8s_window_attention_mfma(void* out, const void* q, long ldq, con
                                          const void* kcache, const void* vcache, const float* kpool, const float* vpool,
                                          const int* block_tables, int max_blocks, const int* cu_q, const int* positions,
                                          int nseq, int max_qlen, int H, int G, int D, int V, int window, int P,
-                                         float scale, int sink, int bs, hipStream_t s) {
+                                         float scale, int sink, int bs, int chunk, float softcap,
+                                         const float* sinkv, int gate_ph, hipStream_t s) {
   if (nseq <= 0 || max_qlen <= 0) return 0;
   if (!k8s_window_mfma_ok(H, G, D, V) || bs <= 0 || nseq > 65535 || G > 65535 || ldq % 8 || ((uintptr_t)q & 15)) return -1;
   if (window > 0 && P > 0 && (kpool == nullptr || vpool == nullptr)) return -1;
@@ -725,7 +779,8 @@ extern "C" int k8s_window_attention_mfma(void* out, const void* q, long ldq, con
 #define K8S_WM_P(NKK, NVB, PF)                                                                                        \
   window_attention_mfma_kernel<NKK, NVB, NCB, PF><<<grid, 256, lds, s>>>(                                             \
       (bf16_t*)out, (const bf16_t*)q, ldq, (const bf16_t*)gate, ldg, (const bf16_t*)kcache, (const bf16_t*)vcache,    \
-      kpool, vpool, block_tables, max_blocks, cu_q, positions, H, G, D, V, window, P, scale, sink, bs, ppb, R)
+      kpool, vpool, block_tables, max_blocks, cu_q, positions, H, G, D, V, window, P, scale, sink, bs, ppb, R, chunk, \
+      softcap, sinkv, gate_ph)
 #define K8S_WM(NKK, NVB)               \
   do {                                 \
     if (pf) K8S_WM_P(NKK, NVB, true);  \

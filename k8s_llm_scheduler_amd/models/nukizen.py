@@ -484,13 +484,15 @@ class NukizenModel(StreamModel):
                                t(get(q + "o")), state=len(self._recurrent))
                 self._recurrent.append(right)
                 mixer = _Side(left, right, t(get(p + "left.out")), t(get(p + "right.out")))
+                if a.kv_from is None:
+                    own_of[i] = left
             w_gu = w_down = None
             if L.ff:
                 w_gu = t(torch.cat([get(f"l{i}.mlp.gate"), get(f"l{i}.mlp.up")]))
                 w_down = t(get(f"l{i}.mlp.down"))
             self.layers.append(_Layer(t(get(f"l{i}.norm1")), mixer, w_gu, w_down))
         for i, L in enumerate(c.layers):       # layers that read another layer's keys and values
-            a = L.mixer if L.type == "attention" else None
+            a = L.mixer if L.type == "attention" else L.mixer[0] if L.type == "parallel" else None
             if a is None or a.kv_from is None:
                 continue
             src = own_of.get(a.kv_from)
@@ -499,7 +501,8 @@ class NukizenModel(StreamModel):
             s = src.cfg
             if (s.kv_heads, s.dim, s.vdim) != (a.kv_heads, a.dim, a.vdim):
                 raise ValueError(f"layer {i}: head sizes differ from layer {a.kv_from}'s, whose cache it reads")
-            self.layers[i].mixer.cache = src.cache
+            w = self.layers[i].mixer
+            (w if isinstance(w, _Attention) else w.left).cache = src.cache
 
     def _weight_roots(self) -> tuple:
         return (self.embed, self.final_norm, self.lm_head, *self.layers)

@@ -209,3 +209,14 @@ def forward(tensors, config, tokens):
     if cap:
         z = float(cap) * torch.tanh(z / float(cap))
     return z, torch.stack(after)
+
+
+def greedy(tensors, config, tokens, n):
+    """n tokens generated greedily after ``tokens`` (the whole sequence is run again for every token)."""
+    toks = list(tokens)
+    out = []
+    for _ in range(n):
+        z, _ = forward(tensors, config, toks)
+        out.append(int(torch.argmax(z[-1])))
+        toks.append(out[-1])
+    return out

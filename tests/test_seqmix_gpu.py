@@ -15,6 +15,9 @@ T = 37
 
 def close(a, b, tol):
     a, b = a.float().cpu(), b.float().cpu()
+    if a.numel() == 0:
+        assert a.shape == b.shape
+        return
     assert (a - b).abs().max().item() <= tol * max(b.abs().max().item(), 1e-6)
 
 
@@ -257,10 +260,13 @@ def test_sigmoid_router_and_plain_combine(E, top):
 
 
 # ----------------------------------------------------------------------------- windowed attention with pooled blocks
-def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0):
+def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0, chunk=0, softcap=0.0, sinks=False, per_head=False,
+                half=False, qk_norm=False, unit=True):
     """Three sequences over shuffled pages: a prompt from 0, a portion that resumes at position 70 and a single token at
     position 130; their earlier tokens are written to the caches first (in two batches, so pooled blocks straddle
-    them)."""
+    them).  ``chunk`` / ``softcap`` / ``sinks`` / ``per_head`` / ``half`` / ``qk_norm`` / ``unit``: the chunked mask,
+    capped scores, learned sinks, one gate number per head, the half rotation layout, whole-projection norms, unit
+    heads."""
     torch.manual_seed(seed)
     nblk = 40
     lens = [(0, 90), (70, 55), (130, 1)]
@@ -285,6 +291,8 @@ def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0):
         return i32(cu), i32(pos), i32(tok_seq), i32(slots)
 
     qb, kb, vb = (torch.randn(n).to(dt) * 0.3 for n in (H * D, G * D, G * V))
+    qnw, knw = ((1.0 + 0.3 * torch.randn(n)).to(dt) if qk_norm else None for n in (H * D, G * D))
+    sv = torch.randn(H) * 2.0 if sinks else None
     e = nblk * sm.pool_entries_per_page(bs, P) if P else 1
     caches = {}
     for dev in ("cpu", DEV):
@@ -302,12 +310,15 @@ def window_case(H, G, D, V, window, P, dims, dt, bs=16, seed=0):
             x = rows(pos.shape[0]).to(dev)
             vfirst = (torch.randn(pos.shape[0], G * V)).to(dev)
             sm.window_kv_write(kc, vc, x, H * D, H * D + G * D, mv(qb), mv(kb), mv(vb), mv(cs), pos.to(dev), slots.to(dev),
-                               H, G, D, V, dims, 1e-6, True, vfirst_in=vfirst, lam=0.3)
+                               H, G, D, V, dims, 1e-6, unit, vfirst_in=vfirst, lam=0.3, half_layout=half, qnw=mv(qnw),
+                               knw=mv(knw))
             sm.window_pool(kp, vp, kc, vc, bt.to(dev), tok_seq.to(dev), pos.to(dev), P, bs)
         goff = H * D + G * D + G * V
-        outs[dev] = (x, sm.window_attention(x, x[:, goff:], kc, vc, kp if P else None, vp if P else None, bt.to(dev),
+        gate = x[:, goff:goff + H] if per_head else x[:, goff:]
+        outs[dev] = (x, sm.window_attention(x, gate, kc, vc, kp if P else None, vp if P else None, bt.to(dev),
                                             tok_seq.to(dev), pos.to(dev), H, window, P, 0.35, True, bs, cu.to(dev),
-                                            max(n for _, n in lens)))
+                                            max(n for _, n in lens), chunk=chunk, softcap=softcap, sinks=mv(sv),
+                                            gate_per_head=per_head))
     return outs, caches
 
 
@@ -339,6 +350,144 @@ def test_window_attention_matrix_cores_match_plain_kernel():
     finally:
         sm.WINDOW_MFMA = old
     close(outs[DEV][1], plain[DEV][1], 2e-2)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,G,D,V,chunk,dims,kw", [
+    (4, 2, 24, 20, 33, 8, dict(softcap=1.5, per_head=True, half=True, unit=False)),       # plain kernel, odd sizes
+    (12, 3, 64, 64, 40, 24, dict(sinks=True, half=True, qk_norm=True, unit=False)),       # matrix cores in bf16
+    (8, 2, 32, 48, 16, 32, dict(softcap=0.8, sinks=True, per_head=True, half=True)),      # chunk = page, full rotation
+    (4, 4, 128, 128, 1, 64, dict(half=True, qk_norm=True)),                                # chunks of one token
+    (6, 2, 16, 16, 1000, 0, dict(per_head=True, sinks=True)),                              # one chunk holds everything
+])
+def test_chunked_attention_variants(dt, tol, H, G, D, V, chunk, dims, kw):
+    """The chunked mask, capped scores, learned sinks, per-head gates, the half rotation layout and whole-projection
+    norms against the reference op, over shuffled pages."""
+    outs, caches = window_case(H, G, D, V, 0, 0, dims, dt, chunk=chunk, **kw)
+    for a, b in zip(caches[DEV][:2], caches["cpu"][:2]):
+        close(a, b, tol)
+    close(outs[DEV][0][:, :H * D], outs["cpu"][0][:, :H * D], tol)
+    close(outs[DEV][1], outs["cpu"][1], tol * 2)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+def test_queries_only_preparation(dt, tol):
+    """A layer that attends another layer's cache prepares its queries and writes no keys or values."""
+    torch.manual_seed(5)
+    H, D, dims = 3, 20, 12
+    x = torch.randn(T, H * D + 5).to(dt)
+    pos = torch.arange(T, dtype=torch.int32)
+    pos[4] = -1
+    cs = ref.rope_table(dims, 64, 500.0)
+    qnw = (1.0 + 0.2 * torch.randn(H * D)).to(dt)
+    xc, xg = x.clone(), x.to(DEV).clone()
+    slots = torch.arange(T, dtype=torch.int32)
+    sm.window_kv_write(None, None, xc, 0, 0, None, None, None, cs, pos, slots, H, 0, D, D, dims, 1e-5, False,
+                       half_layout=True, qnw=qnw)
+    sm.window_kv_write(None, None, xg, 0, 0, None, None, None, cs.to(DEV), pos.to(DEV), slots.to(DEV), H, 0, D, D, dims,
+                       1e-5, False, half_layout=True, qnw=qnw.to(DEV))
+    close(xg, xc, tol)
+    assert torch.equal(xc[4], x[4]) and torch.equal(xg[4].cpu(), x[4])
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+def test_parallel_block_ops(dt, tol):
+    """Two branches in one residual add, the joined norms of two mixers, the relu gate and the soft cap."""
+    torch.manual_seed(6)
+    W = 200
+    x, b1, b2, w = torch.randn(T, W), torch.randn(T, W).to(dt), torch.randn(T, W).to(dt), torch.randn(W).to(dt)
+    xg, xc = x.to(DEV).clone(), x.clone()
+    og = sm.resnorm(xg, w.to(DEV), 1e-5, branch=b1.to(DEV), branch2=b2.to(DEV), out_dtype=dt)
+    oc = sm.resnorm(xc, w, 1e-5, branch=b1, branch2=b2, out_dtype=dt)
+    close(og, oc, tol)
+    close(xg, xc, 1e-6)
+    wa, wb = torch.randn(W).to(dt), torch.randn(W).to(dt)
+    for out in (dt, torch.float32):
+        close(sm.norm_mix(b1.to(DEV), wa.to(DEV), b2.to(DEV), wb.to(DEV), 1e-5, 0.5, 0.25, out),
+              sm.norm_mix(b1, wa, b2, wb, 1e-5, 0.5, 0.25, out), tol)
+    close(sm.norm_mix(b1.to(DEV), wa.to(DEV), None, None, 1e-5, 2.0), sm.norm_mix(b1, wa, None, None, 1e-5, 2.0), tol)
+    a = torch.randn(T, 140).to(dt) * 2
+    close(sm.act(a.to(DEV), sm.ACT_RELU), sm.act(a, sm.ACT_RELU), tol)
+    z = torch.randn(T, 77) * 20
+    close(sm.act(z.to(DEV), sm.ACT_SOFTCAP, limit=12.0), sm.act(z, sm.ACT_SOFTCAP, limit=12.0), 2e-6)
+
+
+# ----------------------------------------------------------------------------- short convolutions, delta rule, RG-LRU
+def _dev(v):
+    return v.to(DEV) if isinstance(v, torch.Tensor) else v
+
+
+@pytest.mark.parametrize("taps,C,unit", [(4, 70, None), (3, 2 * 2 * 24 + 3 * 40, (2 * 2 * 24, 24, 2 * 24, 24 ** -0.5)),
+                                         (1, 33, None), (2, 300, (256, 128, 128, 0.3)), (7, 64, (64, 64, 0, 1.0))])
+def test_short_conv(taps, C, unit):
+    """Convolutions over the batch of `batch()` (an empty sequence, one resumed mid-sequence), twice, so that the second
+    call reads the inputs the first one saved -- also for portions shorter than the taps."""
+    torch.manual_seed(40)
+    cu, pos, slots, tok_seq = batch()
+    w, ib, ob = torch.randn(C, taps), torch.randn(C), torch.randn(C)
+    kw = dict(in_bias=ib, out_bias=ob, act=sm.CONV_SILU if unit else sm.CONV_NONE)
+    if unit:
+        kw.update(unit_cols=unit[0], unit_dim=unit[1], scale_cols=unit[2], scale=unit[3])
+    state = torch.randn(4, max(taps - 1, 0), C)
+    sc, sg = state.clone(), state.to(DEV).clone()
+    x = torch.randn(T, C + 9)[:, 4:4 + C]                 # a view with a row stride
+    for step in range(2):
+        oc = sm.short_conv(x, w, sc, cu, tok_seq, slots, pos, **kw)
+        og = sm.short_conv(x.to(DEV), w.to(DEV), sg, cu.to(DEV), tok_seq.to(DEV), slots.to(DEV), pos.to(DEV),
+                           **{k: _dev(v) for k, v in kw.items()})
+        close(og, oc, 2e-5)
+        close(sg, sc, 1e-6)
+        # next: every sequence goes on by one or two tokens (shorter than the taps)
+        cu = torch.tensor([0, 2, 3, 3, 4], dtype=torch.int32)
+        pos = torch.tensor([9, 10, 6, 30], dtype=torch.int32)
+        tok_seq = torch.tensor([0, 0, 1, 3], dtype=torch.int32)
+        x = torch.randn(4, C)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,G,D,V", [(3, 3, 20, 28), (4, 2, 64, 128), (2, 1, 100, 5), (2, 2, 128, 256), (1, 1, 256, 64),
+                                     (6, 2, 160, 192), (8, 2, 16, 16)])
+def test_delta_scan(dt, tol, H, G, D, V):
+    torch.manual_seed(41)
+    cu, pos, slots, _ = batch()
+    q = torch.nn.functional.normalize(torch.randn(T, G, D), dim=-1) * D ** -0.5
+    k = torch.nn.functional.normalize(torch.randn(T, G, D), dim=-1)
+    qkv = torch.cat([q.reshape(T, -1), k.reshape(T, -1), torch.randn(T, H * V)], 1).contiguous()
+    cols = {"b": 2, "a": 2 + H + 1, "g": 2 + 2 * H + 3}
+    proj = torch.randn(T, cols["g"] + H * V + 2) * 1.5
+    neg_a, dtb, normw = -torch.exp(torch.randn(H) * 0.5), torch.randn(H), 1.0 + 0.2 * torch.randn(V)
+    state = torch.randn(4, H, D * V) * 0.5
+    sc, sg = state.clone(), state.to(DEV).clone()
+    oc = sm.delta_scan(qkv, proj, cols, neg_a, dtb, normw, sc, cu, slots, pos, H, G, D, V, 1e-6, dt)
+    og = sm.delta_scan(qkv.to(DEV), proj.to(DEV), cols, neg_a.to(DEV), dtb.to(DEV), normw.to(DEV), sg, cu.to(DEV),
+                       slots.to(DEV), pos.to(DEV), H, G, D, V, 1e-6, dt)
+    close(og, oc, tol)
+    close(sg, sc, 1e-4)
+    assert torch.equal(sg[1].cpu(), state[1])            # the empty sequence's slot
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("C,blocks,n", [(70, 2, 37), (64, 1, 37), (300, 10, 37), (130, 5, 700)])
+def test_rglru_scan(dt, tol, C, blocks, n):
+    """Short portions (one pass) and a long one (time slices joined exactly), with final states."""
+    torch.manual_seed(42)
+    if n == T:
+        cu, pos, slots, _ = batch()
+    else:
+        cu = torch.tensor([0, n - 40, n - 39, n], dtype=torch.int32)
+        pos = torch.cat([torch.arange(0, n - 40), torch.tensor([17]), torch.arange(5, 44)]).int()
+        slots = torch.tensor([2, 0, 3], dtype=torch.int32)
+    u, gates = torch.randn(n, C), torch.randn(n, blocks, 2 * C // blocks) * 2
+    gb, rate = torch.randn(blocks, 2 * C // blocks), -8.0 * torch.nn.functional.softplus(torch.randn(C))
+    proj, yb = torch.randn(n, C + 7) * 1.5, torch.randn(C)
+    state = torch.randn(4, C)
+    sc, sg = state.clone(), state.to(DEV).clone()
+    mq = int((cu[1:] - cu[:-1]).max())
+    oc = sm.rglru_scan(u, gates, gb, rate, proj, 3, yb, sc, cu, slots, pos, blocks, dt, mq)
+    og = sm.rglru_scan(u.to(DEV), gates.to(DEV), gb.to(DEV), rate.to(DEV), proj.to(DEV), 3, yb.to(DEV), sg, cu.to(DEV),
+                       slots.to(DEV), pos.to(DEV), blocks, dt, mq)
+    close(og, oc, tol)
+    close(sg, sc, 2e-5)
 
 
 # ----------------------------------------------------------------------------- gated matrix-state recurrences

@@ -124,7 +124,10 @@ int k8s_short_conv(float* out, const float* x, long ldx, const float* w, float* 
                    int scale_cols, float scale, float unit_eps, hipStream_t s);
 int k8s_delta_scan(void* out, const float* qkv, const float* proj, long ld, int cb, int ca, int cg, const float* neg_a,
                    const float* dt_bias, const float* normw, float* state, const int* cu_q, const int* seq_slots,
-                   const int* positions, int nseq, int H, int G, int D, int V, float eps, int f32, hipStream_t s);
+                   const int* positions, int nseq, int H, int G, int D, int V, float eps, int f32, int T, int Lc,
+                   float* ws, hipStream_t s);
+int k8s_delta_scan_chunks_ok(int D, int V);
+long long k8s_delta_scan_workspace(int T, int nseq, int H, int D, int V, int Lc);
 int k8s_rglru_scan(void* out, const float* u, const float* gates, const float* gate_bias, const float* rate,
                    const float* proj, long ld, int ycol, const float* ybias, float* state, const int* cu_q,
                    const int* seq_slots, const int* positions, int nseq, int C, int blocks, int max_qlen, int f32,
@@ -469,10 +472,15 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   });
   m.def("delta_scan", [](uintptr_t out, uintptr_t qkv, uintptr_t proj, long ld, int cb, int ca, int cg, uintptr_t neg_a,
                          uintptr_t dt_bias, uintptr_t normw, uintptr_t state, uintptr_t cu_q, uintptr_t seq_slots,
-                         uintptr_t positions, int nseq, int H, int G, int D, int V, float eps, int f32, int64_t s) {
+                         uintptr_t positions, int nseq, int H, int G, int D, int V, float eps, int f32, int T, int Lc,
+                         uintptr_t ws, int64_t s) {
     check(k8s_delta_scan(P(out), P<float>(qkv), P<float>(proj), ld, cb, ca, cg, P<float>(neg_a), P<float>(dt_bias),
                          P<float>(normw), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H,
-                         G, D, V, eps, f32, S(s)), "delta_scan");
+                         G, D, V, eps, f32, T, Lc, P<float>(ws), S(s)), "delta_scan");
+  });
+  m.def("delta_scan_chunks_ok", [](int D, int V) { return k8s_delta_scan_chunks_ok(D, V) != 0; });
+  m.def("delta_scan_workspace", [](int T, int nseq, int H, int D, int V, int Lc) {
+    return k8s_delta_scan_workspace(T, nseq, H, D, V, Lc);
   });
   m.def("rglru_scan", [](uintptr_t out, uintptr_t u, uintptr_t gates, uintptr_t gate_bias, uintptr_t rate,
                          uintptr_t proj, long ld, int ycol, uintptr_t ybias, uintptr_t state, uintptr_t cu_q,

@@ -94,56 +94,88 @@ __global__ void conv_save_kernel(float* __restrict__ state, const float* __restr
     if (r < taps - 1) st[(size_t)r * C + ch] = v[r];
 }
 
-// One workgroup per (sequence, head).  Thread (x, c) owns value column x of the CH key channels [c CH, (c + 1) CH) of
-// S.  Per token every thread forms its channels' part of S^T k and S^T q from the state before the update; the parts
-// meet in LDS (one barrier), then every thread has u for its column and updates its channels, and group c = 0 finishes
-// the output from o = g S_old^T q + (q . k) u, which equals S_new^T q.  The next token's inputs are loaded while the
-// current one is computed; k and q rotate through three LDS rows and the partial sums through two, so one barrier per
-// token orders everything (a second one when the value channels span several waves, for the output's norm).
-// blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest that keeps
-// DX NS within 1024 threads.  qkv rows: [q (G D) | k (G D) | v (H V)].
-template <typename TA, int CH>
+// One workgroup per (sequence or chunk, head).  Thread (x, c) owns value column x of the CH key channels
+// [c CH, (c + 1) CH) of S.  Per token every thread forms its channels' part of S^T k and S^T q from the state before the
+// update; the parts meet in LDS (one barrier), then every thread has u for its column and updates its channels, and
+// group c = 0 finishes the output from o = g S_old^T q + (q . k) u, which equals S_new^T q.  The next token's inputs are
+// loaded while the current one is computed; k and q rotate through three LDS rows and the partial sums through two, so
+// one barrier per token orders everything (a second one when the value channels span several waves, for the output's
+// norm).  blockDim = (DX, NS): DX = the columns rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest
+// that keeps DX NS within 1024 threads.  qkv rows: [q (G D) | k (G D) | v (H V)].
+//
+// MODE 0: a whole portion per workgroup, from the slot's state (zero at position 0) to the slot's state.
+// Long portions run as three passes over chunks of Lc tokens, parallel over chunks.  A token maps S to
+// g (I - beta k k^T) S + beta k v^T, so a chunk maps its start state to P S + L:
+// MODE 1: a chunk run on D + V columns, the first V from zero with the tokens' values (-> L), the other D from the
+//         identity with zero values (-> P, the same update applied to the identity's columns); no outputs; the record
+//         [D][V + D] goes to cs_loc.  delta_prefix_kernel then walks a sequence's chunks, start[c + 1] = P_c start[c] + L_c.
+// MODE 2: a chunk from its start state with outputs; a sequence's last chunk leaves the slot's state.
+template <typename TA, int CH, int MODE>
 __global__ __launch_bounds__(1024) void delta_scan_kernel(
     TA* __restrict__ out, const float* __restrict__ qkv, const float* __restrict__ proj, long ld, int cb, int ca, int cg,
     const float* __restrict__ neg_a, const float* __restrict__ dt_bias, const float* __restrict__ normw,
     float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ seq_slots,
-    const int* __restrict__ positions, int H, int G, int D, int V, float eps) {
+    const int* __restrict__ positions, int H, int G, int D, int V, float eps, int nseq, int Lc,
+    float* __restrict__ cs_loc, const float* __restrict__ cs_start) {
   constexpr int DMAX = 256;
   __shared__ __attribute__((aligned(16))) float sk[3][DMAX], sq[3][DMAX];
   __shared__ float pk[2][1024], pq[2][1024], pqk[2][16];
-  __shared__ float red[4];
-  const int s = blockIdx.x, hd = blockIdx.y;
-  const int a0 = cu_q[s], b0 = cu_q[s + 1];
-  if (b0 <= a0) return;
-  const int p0 = positions[a0];
-  if (p0 < 0) return;
+  __shared__ float red[8];
+  const int hd = blockIdx.y;
+  int s, a0, b0, p0;
+  bool last = true;
+  if (MODE == 0) {
+    s = blockIdx.x;
+    a0 = cu_q[s];
+    b0 = cu_q[s + 1];
+    if (b0 <= a0) return;
+    p0 = positions[a0];
+    if (p0 < 0) return;
+  } else {
+    const WkvChunk ck = wkv_find_chunk(blockIdx.x, cu_q, positions, nseq, Lc);
+    if (ck.s < 0) return;
+    s = ck.s;
+    last = ck.c == ck.n - 1;
+    if (MODE == 1 && last) return;          // nothing follows a sequence's last chunk
+    a0 = cu_q[s] + ck.c * Lc;
+    b0 = min(cu_q[s + 1], a0 + Lc);
+    p0 = positions[a0];
+  }
   const int x = threadIdx.x, c = threadIdx.y, NS = blockDim.y, DX = blockDim.x;
-  const bool onv = x < V, ond = x < D;
+  const int VX = MODE == 1 ? V + D : V;     // columns of this pass
+  const bool onv = x < VX, ond = x < D, isv = x < V;
   const int i0 = c * CH;
   const int gq = hd / (H / G);
   const long row = 2L * G * D + (long)H * V;
   float* st = state + ((size_t)seq_slots[s] * H + hd) * ((size_t)D * V);
+  const size_t lrec = (size_t)D * (V + D), srec = (size_t)D * V;
+  const size_t chunk = (size_t)blockIdx.x * H + hd;
+  // MODE 2 never reads the slot's record, which the sequence's last chunk overwrites: the prefix pass left a copy
+  const float* src = MODE == 2 ? cs_start + chunk * srec : st;
   float S[CH];
 #pragma unroll
-  for (int e = 0; e < CH; ++e) S[e] = (onv && i0 + e < D && p0 != 0) ? st[(size_t)(i0 + e) * V + x] : 0.f;
+  for (int e = 0; e < CH; ++e) {
+    if (MODE == 1) S[e] = (onv && !isv && i0 + e == x - V) ? 1.f : 0.f;
+    else S[e] = (onv && i0 + e < D && p0 != 0) ? src[(size_t)(i0 + e) * V + x] : 0.f;
+  }
   if (c == 0)
     for (int e = x; e < 3 * DMAX; e += DX) (&sk[0][0])[e] = (&sq[0][0])[e] = 0.f;
   const float na = neg_a[hd], dtb = dt_bias[hd];
-  const float nwx = (c == 0 && onv) ? normw[x] : 0.f;
+  const float nwx = (MODE != 1 && c == 0 && onv) ? normw[x] : 0.f;
   float nq = 0.f, nk = 0.f, nv = 0.f, nb = 0.f, nz = 0.f, ng = 0.f;
   auto fetch = [&](int t) {
     if (t >= b0) return;
     const float* r = qkv + (size_t)t * row;
     const float* pr = proj + (size_t)t * ld;
-    if (onv) nv = r[2L * G * D + (long)hd * V + x];
+    if (isv) nv = r[2L * G * D + (long)hd * V + x];
     nb = pr[cb + hd];
     nz = pr[ca + hd];
     if (c == 0) {
       if (ond) {
-        nq = r[(long)gq * D + x];
+        if (MODE != 1) nq = r[(long)gq * D + x];
         nk = r[(long)G * D + (long)gq * D + x];
       }
-      if (onv) ng = pr[cg + (long)hd * V + x];
+      if (MODE != 1 && onv) ng = pr[cg + (long)hd * V + x];
     }
   };
   fetch(a0);
@@ -165,13 +197,17 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         ak[e] = fmaf(k4[e], S[e0 + e], ak[e]);
-        aq[e] = fmaf(q4[e], S[e0 + e], aq[e]);
-        aqk = fmaf(k4[e], q4[e], aqk);
+        if (MODE != 1) {
+          aq[e] = fmaf(q4[e], S[e0 + e], aq[e]);
+          aqk = fmaf(k4[e], q4[e], aqk);
+        }
       }
     }
     pk[pb][c * DX + x] = (ak[0] + ak[1]) + (ak[2] + ak[3]);
-    pq[pb][c * DX + x] = (aq[0] + aq[1]) + (aq[2] + aq[3]);
-    if (x == 0) pqk[pb][c] = aqk;
+    if (MODE != 1) {
+      pq[pb][c * DX + x] = (aq[0] + aq[1]) + (aq[2] + aq[3]);
+      if (x == 0) pqk[pb][c] = aqk;
+    }
     if (c == 0 && ond && t + 1 < b0) {
       sk[nxt][x] = nk;
       sq[nxt][x] = nq;
@@ -190,6 +226,7 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) S[e0 + e] = fmaf(k4[e], u, decay * S[e0 + e]);
     }
+    if (MODE == 1) continue;
     float o = 0.f, ss = 0.f;
     if (c == 0) {
       float qS = 0.f, qk = 0.f;
@@ -211,10 +248,52 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(
       stf(out, (size_t)t * H * V + (size_t)hd * V + x, y);
     }
   }
+  if (MODE == 2 && !last) return;
   if (onv) {
 #pragma unroll
-    for (int e = 0; e < CH; ++e)
-      if (i0 + e < D) st[(size_t)(i0 + e) * V + x] = S[e];
+    for (int e = 0; e < CH; ++e) {
+      if (i0 + e >= D) continue;
+      if (MODE == 1) cs_loc[chunk * lrec + (size_t)(i0 + e) * (V + D) + x] = S[e];
+      else st[(size_t)(i0 + e) * V + x] = S[e];
+    }
+  }
+}
+
+// Start states of a sequence's chunks from the slot's state (zero at position 0) and the chunks' records:
+// start[c + 1] = P_c start[c] + L_c.  One workgroup per (sequence, head); chunk 0 starts from a copy of the slot's record.
+__global__ __launch_bounds__(1024) void delta_prefix_kernel(float* __restrict__ cs_start, const float* __restrict__ cs_loc,
+                                                            const float* __restrict__ state,
+                                                            const int* __restrict__ cu_q,
+                                                            const int* __restrict__ seq_slots,
+                                                            const int* __restrict__ positions, int H, int D, int V,
+                                                            int Lc) {
+  const int s = blockIdx.x, hd = blockIdx.y;
+  int first = 0;
+  for (int y = 0; y < s; ++y) {
+    const int a = cu_q[y], len = cu_q[y + 1] - a;
+    first += (len > 0 && positions[a] >= 0) ? (len + Lc - 1) / Lc : 0;
+  }
+  const int a = cu_q[s], len = cu_q[s + 1] - a;
+  if (len <= 0 || positions[a] < 0) return;
+  const int n = (len + Lc - 1) / Lc;
+  const bool zero = positions[a] == 0;
+  const int DV = D * V, LW = V + D;
+  const float* st = state + ((size_t)seq_slots[s] * H + hd) * DV;
+  float* own = cs_start + ((size_t)first * H + hd) * DV;
+  for (int e = threadIdx.x; e < DV; e += blockDim.x) own[e] = zero ? 0.f : st[e];
+  __syncthreads();
+  for (int c = 0; c + 1 < n; ++c) {
+    const float* cur = cs_start + ((size_t)(first + c) * H + hd) * DV;
+    float* nxt = cs_start + ((size_t)(first + c + 1) * H + hd) * DV;
+    const float* loc = cs_loc + ((size_t)(first + c) * H + hd) * ((size_t)D * LW);
+    for (int e = threadIdx.x; e < DV; e += blockDim.x) {
+      const int i = e / V, x = e - i * V;
+      const float* pr = loc + (size_t)i * LW;
+      float acc = pr[x];
+      for (int j = 0; j < D; ++j) acc = fmaf(pr[V + j], cur[(size_t)j * V + x], acc);
+      nxt[e] = acc;
+    }
+    __syncthreads();                   // the next chunk reads what this one wrote
   }
 }
 
@@ -306,29 +385,72 @@ extern "C" int k8s_short_conv(float* out, const float* x, long ldx, const float*
   return (int)hipGetLastError();
 }
 
+// Block shape for `cols` columns: DX x NS threads with CH key channels per thread; false when it exceeds 1024 threads.
+static bool delta_shape(int D, int cols, int* dx, int* ch) {
+  const int m = D > cols ? D : cols;
+  *dx = (m + 63) / 64 * 64;
+  *ch = 16;
+  while (*ch < 64 && *dx * ((D + *ch - 1) / *ch) > 1024) *ch *= 2;
+  return *dx * ((D + *ch - 1) / *ch) <= 1024;
+}
+
+// Whether portions of these head sizes can run as passes over chunks (the first pass carries D + V columns).
+extern "C" int k8s_delta_scan_chunks_ok(int D, int V) {
+  int dx, ch;
+  return D > 0 && V > 0 && D <= 256 && V <= 256 && delta_shape(D, V + D, &dx, &ch);
+}
+
+// ws (chunked passes): floats for chunks x H records of D (V + D) and of D V, chunks = ceil(T / Lc) + nseq.
+extern "C" long long k8s_delta_scan_workspace(int T, int nseq, int H, int D, int V, int Lc) {
+  if (Lc <= 0) return 0;
+  const long long chunks = (T + Lc - 1) / Lc + nseq;
+  return chunks * H * ((long long)D * (V + D) + (long long)D * V);
+}
+
 extern "C" int k8s_delta_scan(void* out, const float* qkv, const float* proj, long ld, int cb, int ca, int cg,
                               const float* neg_a, const float* dt_bias, const float* normw, float* state,
                               const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int G, int D,
-                              int V, float eps, int f32, hipStream_t s) {
+                              int V, float eps, int f32, int T, int Lc, float* ws, hipStream_t s) {
   if (nseq <= 0) return 0;
   if (H <= 0 || H > 65535 || G <= 0 || H % G || D <= 0 || D > 256 || V <= 0 || V > 256) return -1;
-  const int m = D > V ? D : V, DX = (m + 63) / 64 * 64;
-  int ch = 16;
-  while (ch < 64 && DX * ((D + ch - 1) / ch) > 1024) ch *= 2;
-  if (DX * ((D + ch - 1) / ch) > 1024) return -2;
-  const dim3 block(DX, (D + ch - 1) / ch);
-#define K8S_DS(TA, CH)                                                                                              \
-  delta_scan_kernel<TA, CH><<<dim3(nseq, H), block, 0, s>>>((TA*)out, qkv, proj, ld, cb, ca, cg, neg_a, dt_bias,    \
-                                                            normw, state, cu_q, seq_slots, positions, H, G, D, V, eps)
-#define K8S_DS_T(TA)                  \
-  do {                                \
-    if (ch == 16) K8S_DS(TA, 16);     \
-    else if (ch == 32) K8S_DS(TA, 32); \
-    else K8S_DS(TA, 64);              \
+  int dx, ch;
+  if (!delta_shape(D, V, &dx, &ch)) return -2;
+  dim3 block(dx, (D + ch - 1) / ch);
+  float* loc = nullptr;
+  float* start = nullptr;
+#define K8S_DS(TA, CH, MODE, GX)                                                                                      \
+  delta_scan_kernel<TA, CH, MODE><<<dim3(GX, H), block, 0, s>>>((TA*)out, qkv, proj, ld, cb, ca, cg, neg_a, dt_bias,  \
+                                                                normw, state, cu_q, seq_slots, positions, H, G, D, V, \
+                                                                eps, nseq, Lc, loc, start)
+#define K8S_DS_C(TA, MODE, GX)                 \
+  do {                                         \
+    if (ch == 16) K8S_DS(TA, 16, MODE, GX);    \
+    else if (ch == 32) K8S_DS(TA, 32, MODE, GX); \
+    else K8S_DS(TA, 64, MODE, GX);             \
   } while (0)
-  if (f32) K8S_DS_T(float);
-  else K8S_DS_T(bf16_t);
+#define K8S_DS_T(MODE, GX)                     \
+  do {                                         \
+    if (f32) K8S_DS_C(float, MODE, GX);        \
+    else K8S_DS_C(bf16_t, MODE, GX);           \
+  } while (0)
+  if (Lc <= 0 || ws == nullptr || !k8s_delta_scan_chunks_ok(D, V)) {
+    K8S_DS_T(0, nseq);
+    return (int)hipGetLastError();
+  }
+  const int chunks = (T + Lc - 1) / Lc + nseq;
+  loc = ws;
+  start = ws + (size_t)chunks * H * ((size_t)D * (V + D));
+  const dim3 block2 = block;
+  const int ch2 = ch;
+  delta_shape(D, V + D, &dx, &ch);
+  block = dim3(dx, (D + ch - 1) / ch);
+  K8S_DS_T(1, chunks);
+  delta_prefix_kernel<<<dim3(nseq, H), 1024, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+  block = block2;
+  ch = ch2;
+  K8S_DS_T(2, chunks);
 #undef K8S_DS_T
+#undef K8S_DS_C
 #undef K8S_DS
   return (int)hipGetLastError();
 }

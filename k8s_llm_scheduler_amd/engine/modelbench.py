@@ -1,7 +1,7 @@
 """Prefill and decode throughput of the registered model designs at equal layer sizes (``bench.py --model-bench``).
 
-For every size a Putulorn (dense feed-forwards), a Putulorn with experts, a Rupatar (experts in every layer) and a Llama
-of the same width, depth, feed-forward / expert size and vocabulary are built with random weights and driven through the
+For every size a Putulorn (dense feed-forwards), a Putulorn with experts, a Rupatar (experts in every layer), a Nukizen
+(dense feed-forward beside every mixer) and a Llama of the same width, depth, feed-forward / expert size and vocabulary are built with random weights and driven through the
 same engine entry points:
 
 * prefill: one whole prompt of ``T`` tokens in one step (``LLMEngine.replay_step``, the varlen forward), tokens/s;
@@ -23,12 +23,21 @@ VOCAB = 32768
 
 
 def _register(width: int) -> Dict[str, str]:
-    from ..models import putulorn, rupatar
+    from ..models import nukizen, putulorn, rupatar
     from ..models.config import PRESETS, LlamaConfig
 
     pairs, ff, wd, heads, eff, experts = SIZES[width]
     names = {"putulorn-dense": f"putulorn-w{width}-dense", "putulorn-moe": f"putulorn-w{width}-moe",
-             "rupatar": f"rupatar-w{width}", "llama": f"llama-w{width}"}
+             "rupatar": f"rupatar-w{width}", "nukizen": f"nukizen-w{width}", "llama": f"llama-w{width}"}
+    # Nukizen: 2 x pairs layers in the order attention, parallel (attention + delta rule), rglru, attention on the first
+    # layer's cache; attention shaped like Rupatar's (4 query heads per key head, 128-wide, chunks of 1024), delta-rule
+    # heads of 64 x 64 like the wkv heads, a recurrent unit 5 / 4 of the width in 10 blocks, the dense feed-forward of
+    # the Putulorn-dense layers beside every mixer
+    nukizen.PRESETS[names["nukizen"]] = nukizen.preset(
+        names["nukizen"], width, VOCAB, max(1, pairs // 2), heads=heads, kv_heads=heads // 4, dim=128, vdim=128,
+        chunk=1024, rot_dims=64, side_heads=heads, side_kv_heads=heads // 4, side_dim=128, side_chunk=1024,
+        delta_heads=width // wd, delta_kv_heads=width // wd // 2, delta_dim=wd, delta_vdim=wd, lru_width=width * 5 // 4,
+        lru_blocks=10, ff=ff, order=("attention", "parallel", "rglru", "shared"))
     # Rupatar: 2 x pairs layers in the order attention, hgrn2, attention, mlstm (windowed attention with 4 query heads
     # per key head, window 1024, pooled blocks of 16; recurrences of head size 64 x 64 like the wkv heads), every layer
     # with the experts of the Putulorn-moe layers and a shared expert of the same size

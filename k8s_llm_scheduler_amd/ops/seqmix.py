@@ -631,13 +631,16 @@ def delta_scan_max_dim() -> int:
 
 def delta_scan(qkv: torch.Tensor, proj: torch.Tensor, cols: dict, neg_a: torch.Tensor, dt_bias: torch.Tensor,
                normw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, seq_slots: torch.Tensor,
-               positions: torch.Tensor, H: int, G: int, D: int, V: int, eps: float, out_dtype) -> torch.Tensor:
+               positions: torch.Tensor, H: int, G: int, D: int, V: int, eps: float, out_dtype,
+               chunk: Optional[int] = None) -> torch.Tensor:
     """The gated delta rule with a matrix state per head over a varlen batch.  ``qkv`` fp32 [T, G D | G D | H V]: the
     prepared queries (unit vectors times D^-1/2), keys (unit vectors) and values; ``proj`` fp32 [T, ld] holds the
     columns ``cols`` b (H: beta = sigmoid), a (H: decay = exp(neg_a softplus(a + dt_bias))) and g (H V: output gate,
     silu); ``neg_a`` / ``dt_bias`` / ``normw`` fp32 [H] / [H] / [V].  Per head, with the queries / keys of head
     h // (H / G): S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q; y = o / rms(o) * normw * silu(g).
-    ``state`` [slots, H, D V] fp32 is updated in place (a portion at position 0 starts from zero).  [T, H V]."""
+    ``state`` [slots, H, D V] fp32 is updated in place (a portion at position 0 starts from zero).  [T, H V].
+    Batches of at least SCAN_CHUNK_MIN tokens run as three passes over chunks of SCAN_CHUNK tokens, parallel over chunks
+    (``chunk``: another chunk length, 0: one workgroup per sequence)."""
     T = qkv.shape[0]
     for t, n in ((qkv, "qkv"), (proj, "proj"), (state, "state"), (neg_a, "neg_a"), (dt_bias, "dt_bias"),
                  (normw, "normw")):
@@ -656,10 +659,15 @@ def delta_scan(qkv: torch.Tensor, proj: torch.Tensor, cols: dict, neg_a: torch.T
     if max(D, V) > delta_scan_max_dim():
         raise ValueError(f"delta_scan: head sizes {D} x {V} exceed the kernel's {delta_scan_max_dim()}")
     out = torch.empty(T, H * V, dtype=out_dtype, device=qkv.device)
-    _native().delta_scan(out.data_ptr(), _p(qkv), _p(proj), proj.stride(0), int(cols["b"]), int(cols["a"]),
-                         int(cols["g"]), _p(neg_a), _p(dt_bias), _p(normw), _p(state), _p(cu_q, I32),
-                         _p(seq_slots, I32), _p(positions, I32), cu_q.shape[0] - 1, H, G, D, V, float(eps),
-                         _f32(out_dtype), -1)
+    nat = _native()
+    nseq = cu_q.shape[0] - 1
+    Lc = (SCAN_CHUNK if T >= SCAN_CHUNK_MIN else 0) if chunk is None else int(chunk)
+    if Lc > 0 and not nat.delta_scan_chunks_ok(D, V):
+        Lc = 0
+    ws = torch.empty(nat.delta_scan_workspace(T, nseq, H, D, V, Lc), dtype=F32, device=qkv.device) if Lc > 0 else None
+    nat.delta_scan(out.data_ptr(), _p(qkv), _p(proj), proj.stride(0), int(cols["b"]), int(cols["a"]), int(cols["g"]),
+                   _p(neg_a), _p(dt_bias), _p(normw), _p(state), _p(cu_q, I32), _p(seq_slots, I32), _p(positions, I32),
+                   nseq, H, G, D, V, float(eps), _f32(out_dtype), T, Lc, _p(ws), -1)
     return out
 
 

@@ -464,6 +464,12 @@ def test_delta_scan(dt, tol, H, G, D, V):
     close(og, oc, tol)
     close(sg, sc, 1e-4)
     assert torch.equal(sg[1].cpu(), state[1])            # the empty sequence's slot
+    for chunk in (4, 7, 16, 64):                         # three passes over chunks: same outputs, same final states
+        s2 = state.to(DEV).clone()
+        o2 = sm.delta_scan(qkv.to(DEV), proj.to(DEV), cols, neg_a.to(DEV), dtb.to(DEV), normw.to(DEV), s2, cu.to(DEV),
+                           slots.to(DEV), pos.to(DEV), H, G, D, V, 1e-6, dt, chunk=chunk)
+        close(o2, oc, tol)
+        close(s2, sc, 1e-4)
 
 
 @pytest.mark.parametrize("dt,tol", DTYPES)

@@ -260,13 +260,18 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(
 }
 
 // Start states of a sequence's chunks from the slot's state (zero at position 0) and the chunks' records:
-// start[c + 1] = P_c start[c] + L_c.  One workgroup per (sequence, head); chunk 0 starts from a copy of the slot's record.
+// start[c + 1] = P_c start[c] + L_c.  The value columns are independent, so a workgroup takes (sequence, head, XT value
+// columns): thread (x, i) owns row i of its column; the running columns live in LDS (two buffers), P_c is staged in LDS
+// and the next chunk's P is loaded into registers while the current product runs.  blockDim = (XT, D), XT D <= 1024;
+// dynamic LDS: D (D + 1) + 2 D XT floats.  Chunk 0 starts from a copy of the slot's record.
+template <int NP>
 __global__ __launch_bounds__(1024) void delta_prefix_kernel(float* __restrict__ cs_start, const float* __restrict__ cs_loc,
                                                             const float* __restrict__ state,
                                                             const int* __restrict__ cu_q,
                                                             const int* __restrict__ seq_slots,
                                                             const int* __restrict__ positions, int H, int D, int V,
                                                             int Lc) {
+  extern __shared__ float psm[];
   const int s = blockIdx.x, hd = blockIdx.y;
   int first = 0;
   for (int y = 0; y < s; ++y) {
@@ -277,23 +282,45 @@ __global__ __launch_bounds__(1024) void delta_prefix_kernel(float* __restrict__ 
   if (len <= 0 || positions[a] < 0) return;
   const int n = (len + Lc - 1) / Lc;
   const bool zero = positions[a] == 0;
-  const int DV = D * V, LW = V + D;
+  const int XT = blockDim.x, x = threadIdx.x, i = threadIdx.y;
+  const int col = blockIdx.z * XT + x;
+  const bool ok = col < V;
+  const int DV = D * V, LW = V + D, DP = D + 1;
+  const int tid = i * XT + x, nthr = XT * D;
+  float* Psh = psm;                       // [D][D + 1]
+  float* Ssh = psm + (size_t)D * DP;      // [2][D][XT]
   const float* st = state + ((size_t)seq_slots[s] * H + hd) * DV;
-  float* own = cs_start + ((size_t)first * H + hd) * DV;
-  for (int e = threadIdx.x; e < DV; e += blockDim.x) own[e] = zero ? 0.f : st[e];
-  __syncthreads();
-  for (int c = 0; c + 1 < n; ++c) {
-    const float* cur = cs_start + ((size_t)(first + c) * H + hd) * DV;
-    float* nxt = cs_start + ((size_t)(first + c + 1) * H + hd) * DV;
+  float cur = (ok && !zero) ? st[(size_t)i * V + col] : 0.f;
+  if (ok) cs_start[((size_t)first * H + hd) * DV + (size_t)i * V + col] = cur;
+  Ssh[(size_t)i * XT + x] = cur;
+  float pre[NP];
+  auto load_p = [&](int c) {
     const float* loc = cs_loc + ((size_t)(first + c) * H + hd) * ((size_t)D * LW);
-    for (int e = threadIdx.x; e < DV; e += blockDim.x) {
-      const int i = e / V, x = e - i * V;
-      const float* pr = loc + (size_t)i * LW;
-      float acc = pr[x];
-      for (int j = 0; j < D; ++j) acc = fmaf(pr[V + j], cur[(size_t)j * V + x], acc);
-      nxt[e] = acc;
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+      const int e = tid + k * nthr;
+      pre[k] = e < D * D ? loc[(size_t)(e / D) * LW + V + (e % D)] : 0.f;
     }
-    __syncthreads();                   // the next chunk reads what this one wrote
+  };
+  if (n > 1) load_p(0);
+  for (int c = 0; c + 1 < n; ++c) {
+    const int b = c & 1;
+    __syncthreads();                     // the previous product has read Psh; Ssh[b] is complete
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+      const int e = tid + k * nthr;
+      if (e < D * D) Psh[(size_t)(e / D) * DP + (e % D)] = pre[k];
+    }
+    const float* loc = cs_loc + ((size_t)(first + c) * H + hd) * ((size_t)D * LW);
+    float acc = ok ? loc[(size_t)i * LW + col] : 0.f;
+    __syncthreads();
+    if (c + 2 < n) load_p(c + 1);
+    const float* pr = Psh + (size_t)i * DP;
+    const float* sc = Ssh + (size_t)b * D * XT + x;
+#pragma unroll 8
+    for (int j = 0; j < D; ++j) acc = fmaf(pr[j], sc[(size_t)j * XT], acc);
+    Ssh[(size_t)(b ^ 1) * D * XT + (size_t)i * XT + x] = acc;
+    if (ok) cs_start[((size_t)(first + c + 1) * H + hd) * DV + (size_t)i * V + col] = acc;
   }
 }
 
@@ -397,7 +424,8 @@ static bool delta_shape(int D, int cols, int* dx, int* ch) {
 // Whether portions of these head sizes can run as passes over chunks (the first pass carries D + V columns).
 extern "C" int k8s_delta_scan_chunks_ok(int D, int V) {
   int dx, ch;
-  return D > 0 && V > 0 && D <= 256 && V <= 256 && delta_shape(D, V + D, &dx, &ch);
+  // the prefix pass keeps a chunk's D x D transition in LDS (within 150 KB)
+  return D > 0 && V > 0 && D <= 256 && V <= 256 && delta_shape(D, V + D, &dx, &ch) && (long)D * (D + 1) * 4 <= 150 * 1024;
 }
 
 // ws (chunked passes): floats for chunks x H records of D (V + D) and of D V, chunks = ceil(T / Lc) + nseq.
@@ -445,7 +473,25 @@ extern "C" int k8s_delta_scan(void* out, const float* qkv, const float* proj, lo
   delta_shape(D, V + D, &dx, &ch);
   block = dim3(dx, (D + ch - 1) / ch);
   K8S_DS_T(1, chunks);
-  delta_prefix_kernel<<<dim3(nseq, H), 1024, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+  {
+    int xt = 16;
+    while (xt > 1 && xt * D > 1024) xt /= 2;
+    const dim3 pgrid(nseq, H, (V + xt - 1) / xt), pblock(xt, D);
+    const size_t plds = ((size_t)D * (D + 1) + 2 * (size_t)D * xt) * sizeof(float);
+    const int np = (D * D + xt * D - 1) / (xt * D);     // elements of P per thread: D / xt
+#define K8S_DP(NP)                                                                                                     \
+  do {                                                                                                                 \
+    if (plds > 48 * 1024 &&                                                                                            \
+        hipFuncSetAttribute((const void*)delta_prefix_kernel<NP>, hipFuncAttributeMaxDynamicSharedMemorySize,          \
+                            (int)plds) != hipSuccess)                                                                  \
+      return -3;                                                                                                       \
+    delta_prefix_kernel<NP><<<pgrid, pblock, plds, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);   \
+  } while (0)
+    if (np <= 4) K8S_DP(4);
+    else if (np <= 16) K8S_DP(16);
+    else K8S_DP(64);
+#undef K8S_DP
+  }
   block = block2;
   ch = ch2;
   K8S_DS_T(2, chunks);

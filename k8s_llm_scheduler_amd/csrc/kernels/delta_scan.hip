@@ -16,8 +16,8 @@ namespace k8sllm {
 
 constexpr int CONV_MAX_TAPS = 16;
 
-// One workgroup per token.  The first unit_cols channels go one wave per group of unit_dim (<= 256) channels, the
-// rest one thread per channel.
+// Workgroups (token, slice of the channels).  The first unit_cols channels go one wave per group of unit_dim (<= 256)
+// channels, the rest one thread per channel; the slices of a token share both lists.
 __global__ __launch_bounds__(256) void short_conv_kernel(
     float* __restrict__ out, const float* __restrict__ x, long ldx, const float* __restrict__ w,
     const float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ tok_seq,
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
   float* dst = out + (size_t)t * C;
   const int ngroups = unit_dim > 0 ? unit_cols / unit_dim : 0;
-  for (int gv = wave; gv < ngroups; gv += nw) {
+  for (int gv = blockIdx.y * nw + wave; gv < ngroups; gv += nw * gridDim.y) {
     float y[4], ss = 0.f;
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
@@ -63,7 +63,8 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
       if (d < unit_dim) dst[ch] = y[n] * inv * (ch < scale_cols ? scale : 1.f);
     }
   }
-  for (int ch = ngroups * unit_dim + tid; ch < C; ch += blockDim.x) dst[ch] = value(ch) * (ch < scale_cols ? scale : 1.f);
+  for (int ch = ngroups * unit_dim + blockIdx.y * blockDim.x + tid; ch < C; ch += blockDim.x * gridDim.y)
+    dst[ch] = value(ch) * (ch < scale_cols ? scale : 1.f);
 }
 
 // state[slot of s] <- the last taps - 1 inputs of sequence s after this portion (a portion shorter than that keeps the
@@ -402,8 +403,13 @@ extern "C" int k8s_short_conv(float* out, const float* x, long ldx, const float*
   if (taps > 1 && state == nullptr) return -1;
   if (unit_cols < 0 || unit_cols > C || (unit_cols > 0 && (unit_dim <= 0 || unit_dim > 256 || unit_cols % unit_dim)))
     return -1;
-  short_conv_kernel<<<T, 256, 0, s>>>(out, x, ldx, w, state, cu_q, tok_seq, seq_slots, positions, in_bias, out_bias, act,
-                                      C, taps, unit_cols, unit_dim, scale_cols, scale, unit_eps);
+  // few tokens (decoding): the channels of a token are spread over several workgroups
+  const int ngroups = unit_cols > 0 ? unit_cols / unit_dim : 0;
+  int ny = (ngroups + 3) / 4 > (C - unit_cols + 255) / 256 ? (ngroups + 3) / 4 : (C - unit_cols + 255) / 256;
+  const int want = T >= 1024 ? 1 : (1024 + T - 1) / T;
+  ny = ny < 1 ? 1 : (ny > want ? want : ny);
+  short_conv_kernel<<<dim3(T, ny), 256, 0, s>>>(out, x, ldx, w, state, cu_q, tok_seq, seq_slots, positions, in_bias,
+                                                out_bias, act, C, taps, unit_cols, unit_dim, scale_cols, scale, unit_eps);
   if (taps > 1) {
     const dim3 grid(nseq, (C + 255) / 256);
     if (grid.y > 65535) return -2;

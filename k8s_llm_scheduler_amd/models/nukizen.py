@@ -275,18 +275,18 @@ def preset(name: str, width: int, vocab: int, repeats: int, *, heads: int, kv_he
                 if src is None:
                     first = len(layers)
                 mixer: object = AttentionConfig(heads, kv_heads, dim, vdim, 1.0 / math.sqrt(dim), chunk=chunk,
-                                                rot_dims=rot_dims, rot_base=20000.0, softcap=30.0, kv_from=src, gate=True)
+                                                rot_dims=rot_dims, rot_base=10000.0, softcap=50.0, kv_from=src, gate=True)
                 layers.append(LayerConfig("attention", mixer, ff))
             elif kind == "rglru":
                 layers.append(LayerConfig("rglru", RglruConfig(lru_width, lru_blocks, 4), ff))
             else:
                 left = AttentionConfig(side_heads, side_kv_heads, side_dim, side_dim, 1.0 / math.sqrt(side_dim),
-                                       chunk=side_chunk, rot_dims=side_dim, rot_base=20000.0,
-                                       rot_scaling={"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0},
+                                       chunk=side_chunk, rot_dims=side_dim, rot_base=10000.0,
+                                       rot_scaling={"factor": 8.0, "original": 2048, "fast": 16.0, "slow": 2.0},
                                        qk_norm=True, sink=True)
                 layers.append(LayerConfig("parallel", (left, DeltaConfig(delta_heads, delta_kv_heads, delta_dim,
                                                                          delta_vdim, 3)), ff))
-    return NukizenConfig(name, vocab, width, layers, rms_eps=1e-5, logit_softcap=30.0)
+    return NukizenConfig(name, vocab, width, layers, rms_eps=1e-6, logit_softcap=40.0)
 
 
 PRESETS = {

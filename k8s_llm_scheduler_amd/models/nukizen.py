@@ -141,7 +141,7 @@ def _layer_from(l: dict) -> LayerConfig:
                  DeltaConfig(int(r["heads"]), int(r.get("kv_heads") or r["heads"]), int(r["dim"]),
                              int(r.get("vdim") or r["dim"]), int(r.get("conv") or 1)))
     else:
-        raise ValueError(f"unknown mixer type {kind!r}")
+        raise ValueError(f"unknown mixer type {kind!r} (known: {', '.join(MIXERS)})")
     mlp = l.get("mlp")
     if mlp is not None and mlp.get("kind", "dense") != "dense":
         raise ValueError(f"unknown mlp kind {mlp['kind']!r}")

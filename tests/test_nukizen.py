@@ -5,7 +5,6 @@ Small own configurations, random weights; where random weights would hide a faul
 shows."""
 
 import copy
-import math
 
 import pytest
 import torch

@@ -116,12 +116,16 @@ int k8s_embed_rows(float* out, const int* ids, const void* table, int T, int W, 
                    hipStream_t s);
 int k8s_resnorm(float* x, const void* branch, const void* branch2, float mult, const void* rowvec, const void* w,
                 float offset, float eps, void* out, int T, int W, int groups, int f32, hipStream_t s);
-int k8s_norm_mix(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, float ca, float cb,
-                 int T, int W, int in_f32, int out_f32, hipStream_t s);
-int k8s_short_conv(float* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
+int k8s_norm_mix(void* out, const void* a, long lda, const void* wa, const void* b, const void* wb, float eps, float ca,
+                 float cb, int T, int W, int groups, int in_f32, int out_f32, hipStream_t s);
+int k8s_postnorm(float* x, const void* branch, const void* branch2, float alpha, float c1, float c2, float gain,
+                 float eps, void* out, int T, int W, int f32, hipStream_t s);
+int k8s_gate_mul(void* out, const void* y, long ldy, const void* gate, long ldg, int T, int F, int kind, int y_f32,
+                 int f32, hipStream_t s);
+int k8s_short_conv(void* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
                    const int* tok_seq, const int* seq_slots, const int* positions, const float* in_bias,
                    const float* out_bias, int act, int T, int C, int taps, int nseq, int unit_cols, int unit_dim,
-                   int scale_cols, float scale, float unit_eps, hipStream_t s);
+                   int scale_cols, float scale, float unit_eps, int residual, int out_f32, hipStream_t s);
 int k8s_delta_scan(void* out, const float* qkv, const float* proj, long ld, int cb, int ca, int cg, const float* neg_a,
                    const float* dt_bias, const float* normw, float* state, const int* cu_q, const int* seq_slots,
                    const int* positions, int nseq, int H, int G, int D, int V, float eps, int f32, int T, int Lc,
@@ -149,22 +153,22 @@ int k8s_wkv_scan(void* out, const void* r, const void* k, const void* v, const v
                  hipStream_t s);
 int k8s_latent_kv_write(void* cache, const void* dkv, const void* normw, void* q, const float* cos_sin,
                         const int* positions, const int* slot_mapping, int T, int C, int R, int H, int Dn, int dims,
-                        float eps, int f32, hipStream_t s);
+                        float eps, int f32, long ldd, int interleaved, hipStream_t s);
 int k8s_latent_attention(void* out, const void* q_abs, const void* q, const void* cache, const int* block_tables,
                          int max_blocks, const int* tok_seq, const int* positions, int T, int C, int R, int H, int Dn,
-                         int window, float scale, int bs, int f32, hipStream_t s);
+                         int window, float scale, int bs, int f32, const float* sinks, hipStream_t s);
 int k8s_latent_mfma_ok(int C, int R, int Dn);
 int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, const void* q_abs, const void* q, const void* cache,
                               const int* block_tables, int max_blocks, const int* tok_seq, const int* positions, int T,
                               int C, int R, int H, int Dn, int window, float scale, int bs, int nsplit, const int* cu_q,
-                              int nseq, int max_qlen, hipStream_t s);
+                              int nseq, int max_qlen, const float* sinks, hipStream_t s);
 int k8s_moe_route(int* idx, float* w, const float* logits, int ld, int T, int E, int top, float scale, int mode,
                   hipStream_t s);
 int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long ld, int koff, int voff, const void* qb,
                         const void* kb, const void* vb, const float* cos_sin, const int* positions,
                         const int* slot_mapping, const float* vfirst_in, float* vfirst_out, float lam, int T, int H, int G,
                         int D, int V, int dims, float eps, int unit, int half_layout, const void* qnw, const void* knw,
-                        int f32, hipStream_t s);
+                        const void* hqw, const void* hkw, int f32, hipStream_t s);
 int k8s_window_pool(float* kpool, float* vpool, const void* kcache, const void* vcache, const int* block_tables,
                     int max_blocks, const int* tok_seq, const int* positions, int T, int G, int D, int V, int P, int bs,
                     int f32, hipStream_t s);
@@ -185,7 +189,8 @@ long long k8s_gated_scan_record(int kind, int D, int V);
 int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf, int cg,
                    const void* fbias, const void* ibias, const void* lower, const void* normw, float* state,
                    const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H, int D, int V, float eps,
-                   float cap, int f32, int T, int Lc, float* ws, hipStream_t s);
+                   float cap, int f32, int T, int Lc, float* ws, const float* aux, long ldaux, const float* hpar, int R,
+                   hipStream_t s);
 long long k8s_gated_scan_workspace(int T, int nseq, int H, int D, int V, int Lc);
 int k8s_moe_align(int* sorted_tok, int* pos_of_pair, int* seg, int* tiles, int ntiles, const int* topk_idx, int P,
                   int top, int E, int BM, hipStream_t s);
@@ -457,18 +462,29 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
     check(k8s_resnorm(P<float>(x), P(branch), P(branch2), mult, P(rowvec), P(w), offset, eps, P(out), T, W, groups, f32,
                       S(s)), "resnorm");
   });
-  m.def("norm_mix", [](uintptr_t out, uintptr_t a, uintptr_t wa, uintptr_t b, uintptr_t wb, float eps, float ca,
-                       float cb, int T, int W, int in_f32, int out_f32, int64_t s) {
-    check(k8s_norm_mix(P(out), P(a), P(wa), P(b), P(wb), eps, ca, cb, T, W, in_f32, out_f32, S(s)), "norm_mix");
+  m.def("norm_mix", [](uintptr_t out, uintptr_t a, long lda, uintptr_t wa, uintptr_t b, uintptr_t wb, float eps,
+                       float ca, float cb, int T, int W, int groups, int in_f32, int out_f32, int64_t s) {
+    check(k8s_norm_mix(P(out), P(a), lda, P(wa), P(b), P(wb), eps, ca, cb, T, W, groups, in_f32, out_f32, S(s)),
+          "norm_mix");
+  });
+  m.def("postnorm", [](uintptr_t x, uintptr_t branch, uintptr_t branch2, float alpha, float c1, float c2, float gain,
+                       float eps, uintptr_t out, int T, int W, int f32, int64_t s) {
+    check(k8s_postnorm(P<float>(x), P(branch), P(branch2), alpha, c1, c2, gain, eps, P(out), T, W, f32, S(s)),
+          "postnorm");
+  });
+  m.def("gate_mul", [](uintptr_t out, uintptr_t y, long ldy, uintptr_t gate, long ldg, int T, int F, int kind,
+                       int y_f32, int f32, int64_t s) {
+    check(k8s_gate_mul(P(out), P(y), ldy, P(gate), ldg, T, F, kind, y_f32, f32, S(s)), "gate_mul");
   });
   // short convolutions, the gated delta rule, the real-gated linear recurrent unit (delta_scan.hip)
   m.def("short_conv", [](uintptr_t out, uintptr_t x, long ldx, uintptr_t w, uintptr_t state, uintptr_t cu_q,
                          uintptr_t tok_seq, uintptr_t seq_slots, uintptr_t positions, uintptr_t in_bias,
                          uintptr_t out_bias, int act, int T, int C, int taps, int nseq, int unit_cols, int unit_dim,
-                         int scale_cols, float scale, float unit_eps, int64_t s) {
-    check(k8s_short_conv(P<float>(out), P<float>(x), ldx, P<float>(w), P<float>(state), P<int>(cu_q), P<int>(tok_seq),
+                         int scale_cols, float scale, float unit_eps, int residual, int out_f32, int64_t s) {
+    check(k8s_short_conv(P(out), P<float>(x), ldx, P<float>(w), P<float>(state), P<int>(cu_q), P<int>(tok_seq),
                          P<int>(seq_slots), P<int>(positions), P<float>(in_bias), P<float>(out_bias), act, T, C, taps,
-                         nseq, unit_cols, unit_dim, scale_cols, scale, unit_eps, S(s)), "short_conv");
+                         nseq, unit_cols, unit_dim, scale_cols, scale, unit_eps, residual, out_f32, S(s)),
+          "short_conv");
   });
   m.def("delta_scan", [](uintptr_t out, uintptr_t qkv, uintptr_t proj, long ld, int cb, int ca, int cg, uintptr_t neg_a,
                          uintptr_t dt_bias, uintptr_t normw, uintptr_t state, uintptr_t cu_q, uintptr_t seq_slots,
@@ -522,24 +538,27 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("wkv_workspace", [](int T, int nseq, int H, int D, int Lc) { return k8s_wkv_workspace(T, nseq, H, D, Lc); });
   m.def("latent_kv_write", [](uintptr_t cache, uintptr_t dkv, uintptr_t normw, uintptr_t q, uintptr_t cos_sin,
                               uintptr_t positions, uintptr_t slots, int T, int C, int R, int H, int Dn, int dims,
-                              float eps, int f32, int64_t s) {
+                              float eps, int f32, long ldd, int interleaved, int64_t s) {
     check(k8s_latent_kv_write(P(cache), P(dkv), P(normw), P(q), P<float>(cos_sin), P<int>(positions), P<int>(slots), T,
-                              C, R, H, Dn, dims, eps, f32, S(s)), "latent_kv_write");
+                              C, R, H, Dn, dims, eps, f32, ldd, interleaved, S(s)), "latent_kv_write");
   });
   m.def("latent_attention", [](uintptr_t out, uintptr_t q_abs, uintptr_t q, uintptr_t cache, uintptr_t bt,
                                int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int C, int R, int H,
-                               int Dn, int window, float scale, int bs, int f32, int64_t s) {
+                               int Dn, int window, float scale, int bs, int f32, uintptr_t sinks, int64_t s) {
     check(k8s_latent_attention(P(out), P(q_abs), P(q), P(cache), P<int>(bt), max_blocks, P<int>(tok_seq),
-                               P<int>(positions), T, C, R, H, Dn, window, scale, bs, f32, S(s)), "latent_attention");
+                               P<int>(positions), T, C, R, H, Dn, window, scale, bs, f32, P<float>(sinks), S(s)),
+          "latent_attention");
   });
   m.def("latent_mfma_ok", [](int C, int R, int Dn) { return k8s_latent_mfma_ok(C, R, Dn) != 0; });
   m.def("latent_attention_mfma", [](uintptr_t out, uintptr_t pacc, uintptr_t pml, uintptr_t q_abs, uintptr_t q,
                                     uintptr_t cache, uintptr_t bt, int max_blocks, uintptr_t tok_seq,
                                     uintptr_t positions, int T, int C, int R, int H, int Dn, int window, float scale,
-                                    int bs, int nsplit, uintptr_t cu_q, int nseq, int max_qlen, int64_t s) {
+                                    int bs, int nsplit, uintptr_t cu_q, int nseq, int max_qlen, uintptr_t sinks,
+                                    int64_t s) {
     check(k8s_latent_attention_mfma(P(out), P<float>(pacc), P<float>(pml), P(q_abs), P(q), P(cache), P<int>(bt),
                                     max_blocks, P<int>(tok_seq), P<int>(positions), T, C, R, H, Dn, window, scale, bs,
-                                    nsplit, P<int>(cu_q), nseq, max_qlen, S(s)), "latent_attention_mfma");
+                                    nsplit, P<int>(cu_q), nseq, max_qlen, P<float>(sinks), S(s)),
+          "latent_attention_mfma");
   });
   m.def("moe_route", [](uintptr_t idx, uintptr_t w, uintptr_t logits, int ld, int T, int E, int top, float scale,
                         int mode, int64_t s) {
@@ -551,10 +570,11 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
                               uintptr_t qb, uintptr_t kb, uintptr_t vb, uintptr_t cos_sin, uintptr_t positions,
                               uintptr_t slots, uintptr_t vfirst_in, uintptr_t vfirst_out, float lam, int T, int H, int G,
                               int D, int V, int dims, float eps, int unit, int half_layout, uintptr_t qnw,
-                              uintptr_t knw, int f32, int64_t s) {
+                              uintptr_t knw, uintptr_t hqw, uintptr_t hkw, int f32, int64_t s) {
     check(k8s_window_kv_write(P(kcache), P(vcache), P(qkv), ld, koff, voff, P(qb), P(kb), P(vb), P<float>(cos_sin),
                               P<int>(positions), P<int>(slots), P<float>(vfirst_in), P<float>(vfirst_out), lam, T, H, G,
-                              D, V, dims, eps, unit, half_layout, P(qnw), P(knw), f32, S(s)), "window_kv_write");
+                              D, V, dims, eps, unit, half_layout, P(qnw), P(knw), P(hqw), P(hkw), f32, S(s)),
+          "window_kv_write");
   });
   m.def("window_pool", [](uintptr_t kpool, uintptr_t vpool, uintptr_t kcache, uintptr_t vcache, uintptr_t bt,
                           int max_blocks, uintptr_t tok_seq, uintptr_t positions, int T, int G, int D, int V, int P_,
@@ -590,10 +610,12 @@ PYBIND11_MODULE(K8S_MODULE_NAME, m) {
   m.def("gated_scan", [](uintptr_t out, uintptr_t proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf,
                          int cg, uintptr_t fbias, uintptr_t ibias, uintptr_t lower, uintptr_t normw, uintptr_t state,
                          uintptr_t cu_q, uintptr_t seq_slots, uintptr_t positions, int nseq, int H, int D, int V,
-                         float eps, float cap, int f32, int T, int Lc, uintptr_t ws, int64_t s) {
+                         float eps, float cap, int f32, int T, int Lc, uintptr_t ws, uintptr_t aux, long ldaux,
+                         uintptr_t hpar, int R, int64_t s) {
     check(k8s_gated_scan(P(out), P<float>(proj), ld, kind, cq, ck, cv, ci, cf, cg, P(fbias), P(ibias), P(lower),
                          P(normw), P<float>(state), P<int>(cu_q), P<int>(seq_slots), P<int>(positions), nseq, H, D, V,
-                         eps, cap, f32, T, Lc, P<float>(ws), S(s)), "gated_scan");
+                         eps, cap, f32, T, Lc, P<float>(ws), P<float>(aux), ldaux, P<float>(hpar), R, S(s)),
+          "gated_scan");
   });
   m.def("gated_scan_workspace", [](int T, int nseq, int H, int D, int V, int Lc) {
     return k8s_gated_scan_workspace(T, nseq, H, D, V, Lc);

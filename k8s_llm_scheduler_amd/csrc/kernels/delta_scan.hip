@@ -17,13 +17,16 @@ namespace k8sllm {
 constexpr int CONV_MAX_TAPS = 16;
 
 // Workgroups (token, slice of the channels).  The first unit_cols channels go one wave per group of unit_dim (<= 256)
-// channels, the rest one thread per channel; the slices of a token share both lists.
+// channels, the rest one thread per channel; the slices of a token share both lists.  `residual`: the token's own input
+// is added to the result (y = x + conv(x), after bias and activation).  TO: the output's type (fp32, or bf16 for a
+// convolution whose result feeds a bf16 projection).
+template <typename TO>
 __global__ __launch_bounds__(256) void short_conv_kernel(
-    float* __restrict__ out, const float* __restrict__ x, long ldx, const float* __restrict__ w,
+    TO* __restrict__ out, const float* __restrict__ x, long ldx, const float* __restrict__ w,
     const float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ tok_seq,
     const int* __restrict__ seq_slots, const int* __restrict__ positions, const float* __restrict__ in_bias,
     const float* __restrict__ out_bias, int act, int C, int taps, int unit_cols, int unit_dim, int scale_cols,
-    float scale, float unit_eps) {
+    float scale, float unit_eps, int residual) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   if (pos < 0) return;
@@ -42,10 +45,11 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
       acc = fmaf(w[(size_t)ch * taps + j], xv, acc);
     }
     if (act == 1) acc = acc / (1.f + expf(-acc));
+    if (residual) acc += x[(size_t)t * ldx + ch] + ib;
     return acc;
   };
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
-  float* dst = out + (size_t)t * C;
+  TO* dst = out + (size_t)t * C;
   const int ngroups = unit_dim > 0 ? unit_cols / unit_dim : 0;
   for (int gv = blockIdx.y * nw + wave; gv < ngroups; gv += nw * gridDim.y) {
     float y[4], ss = 0.f;
@@ -60,11 +64,11 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       const int d = lane + 64 * n, ch = gv * unit_dim + d;
-      if (d < unit_dim) dst[ch] = y[n] * inv * (ch < scale_cols ? scale : 1.f);
+      if (d < unit_dim) stf(dst, ch, y[n] * inv * (ch < scale_cols ? scale : 1.f));
     }
   }
   for (int ch = ngroups * unit_dim + blockIdx.y * blockDim.x + tid; ch < C; ch += blockDim.x * gridDim.y)
-    dst[ch] = value(ch) * (ch < scale_cols ? scale : 1.f);
+    stf(dst, ch, value(ch) * (ch < scale_cols ? scale : 1.f));
 }
 
 // state[slot of s] <- the last taps - 1 inputs of sequence s after this portion (a portion shorter than that keeps the
@@ -394,10 +398,11 @@ __global__ __launch_bounds__(1024) void rglru_scan_kernel(
 
 using namespace k8sllm;
 
-extern "C" int k8s_short_conv(float* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
+extern "C" int k8s_short_conv(void* out, const float* x, long ldx, const float* w, float* state, const int* cu_q,
                               const int* tok_seq, const int* seq_slots, const int* positions, const float* in_bias,
                               const float* out_bias, int act, int T, int C, int taps, int nseq, int unit_cols,
-                              int unit_dim, int scale_cols, float scale, float unit_eps, hipStream_t s) {
+                              int unit_dim, int scale_cols, float scale, float unit_eps, int residual, int out_f32,
+                              hipStream_t s) {
   if (T <= 0 || nseq <= 0) return 0;
   if (C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || act < 0 || act > 1) return -1;
   if (taps > 1 && state == nullptr) return -1;
@@ -408,8 +413,14 @@ extern "C" int k8s_short_conv(float* out, const float* x, long ldx, const float*
   int ny = (ngroups + 3) / 4 > (C - unit_cols + 255) / 256 ? (ngroups + 3) / 4 : (C - unit_cols + 255) / 256;
   const int want = T >= 1024 ? 1 : (1024 + T - 1) / T;
   ny = ny < 1 ? 1 : (ny > want ? want : ny);
-  short_conv_kernel<<<dim3(T, ny), 256, 0, s>>>(out, x, ldx, w, state, cu_q, tok_seq, seq_slots, positions, in_bias,
-                                                out_bias, act, C, taps, unit_cols, unit_dim, scale_cols, scale, unit_eps);
+  if (out_f32)
+    short_conv_kernel<float><<<dim3(T, ny), 256, 0, s>>>((float*)out, x, ldx, w, state, cu_q, tok_seq, seq_slots,
+                                                         positions, in_bias, out_bias, act, C, taps, unit_cols, unit_dim,
+                                                         scale_cols, scale, unit_eps, residual);
+  else
+    short_conv_kernel<bf16_t><<<dim3(T, ny), 256, 0, s>>>((bf16_t*)out, x, ldx, w, state, cu_q, tok_seq, seq_slots,
+                                                          positions, in_bias, out_bias, act, C, taps, unit_cols,
+                                                          unit_dim, scale_cols, scale, unit_eps, residual);
   if (taps > 1) {
     const dim3 grid(nseq, (C + 255) / 256);
     if (grid.y > 65535) return -2;

@@ -7,6 +7,12 @@
 //       i = cap tanh((zi + bi) / cap), f = logsigmoid(cap tanh((zf + bf) / cap))  per head;
 //       m' = max(f + m, i), a = exp(f + m - m'), b = exp(i - m');  S <- a S + b k v^T, n <- a n + b k;
 //       o = S^T q / (max(|n . q|, exp(-m')) + 1e-6), q = zq / sqrt(D);  y = o / rms(o) * normw[H V] * sigmoid(zg)
+//   KIND 2 (state-space duality: one decay per head and token, set by a step size)
+//       dt = softplus(zdt + dt_bias), a = exp(neg_a dt) with neg_a = -exp(A_log) per head;  S <- a S + dt B x^T;
+//       y = (S^T C + skip x) * silu(zg);  B and C [D] are shared by the R heads of a group, x [V] is the head's own;
+//       no norm here (it runs over groups of heads afterwards) and y is stored in fp32.  x, B and C come from `proj`
+//       (the convolved branch), zdt and zg from `aux` (the input projection); neg_a, dt_bias and skip from `hpar`
+//       ([3][H] fp32).
 // Everything that enters the recurrence (gates, decays, state, norms) is fp32: the kernels read the fused input
 // projection as fp32 [T, ld] with the parts at column offsets, and write y in the activation type.
 // Varlen batches: sequence s owns tokens cu_q[s] .. cu_q[s + 1] - 1 and the state record of slot seq_slots[s]; a portion
@@ -44,7 +50,9 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
                                                           const int* __restrict__ positions, int H, int D, int V,
                                                           float eps, float cap, int nseq, int Lc,
                                                           float* __restrict__ cs_loc,
-                                                          const float* __restrict__ cs_start) {
+                                                          const float* __restrict__ cs_start,
+                                                          const float* __restrict__ aux, long ldaux,
+                                                          const float* __restrict__ hpar, int R) {
   constexpr int DMAX = 256;
   __shared__ __attribute__((aligned(16))) float sq[DMAX], sa[DMAX], sb[DMAX];
   __shared__ float po[DMAX / CH][DMAX];
@@ -94,7 +102,13 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
   if (c == 0)
     for (int e = x; e < DMAX; e += DX) sq[e] = sa[e] = sb[e] = 0.f;
   float lowx = 0.f, fbx = 0.f, nwx = 0.f, fbh = 0.f, ibh = 0.f;
-  if (KIND == 0) {
+  float nega = 0.f, skip = 0.f;
+  const int qk0 = KIND == 2 ? (hd / R) * D : hd * D;    // the head's (KIND 2: its group's) query / key columns
+  if (KIND == 2) {
+    nega = hpar[hd];
+    fbh = hpar[H + hd];
+    skip = hpar[2 * H + hd];
+  } else if (KIND == 0) {
     if (c == 0 && ond) {
       lowx = ldf(lower, (size_t)hd * D + x);
       fbx = fbias != nullptr ? ldf(fbias, (size_t)hd * D + x) : 0.f;
@@ -113,6 +127,16 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
     if (t >= b0) return;
     const float* r = proj + (size_t)t * ld;
     if (onv) nv = r[co.v + (size_t)hd * V + x];
+    if (KIND == 2) {
+      const float* ar = aux + (size_t)t * ldaux;
+      nf = ar[co.f + hd];
+      if (MODE != 1 && c == 0 && onv) ng = ar[co.g + (size_t)hd * V + x];
+      if (c == 0 && ond) {
+        if (MODE != 1) nq = r[co.q + qk0 + x];
+        nk = r[co.k + qk0 + x];
+      }
+      return;
+    }
     if (KIND == 1) {
       nf = r[co.f + hd];
       ni = r[co.i + hd];
@@ -128,8 +152,16 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
   for (int t = a0; t < b0; ++t) {
     const float cq = nq, ck = nk, cv = nv, cf = nf, ci = ni, cg = ng;
     fetch(t + 1);
-    float ka = 1.f;   // KIND 1: the head's keep factor
-    if (KIND == 0) {
+    float ka = 1.f;   // KIND 1, 2: the head's keep factor
+    if (KIND == 2) {
+      const float zd = cf + fbh;
+      const float dt = fmaxf(zd, 0.f) + log1pf(expf(-fabsf(zd)));
+      ka = expf(nega * dt);
+      if (c == 0 && ond) {
+        sq[x] = cq;
+        sb[x] = dt * ck;
+      }
+    } else if (KIND == 0) {
       if (c == 0 && ond) {
         const float f = lowx + (1.f - lowx) / (1.f + expf(-(cf + fbx)));
         sq[x] = cq / (1.f + expf(-cq));
@@ -172,7 +204,7 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       for (int e = 0; e < 4; ++e) {
         S[e0 + e] = fmaf(a4[e], S[e0 + e], b4[e] * cv);
         if (MODE != 1) o4[e] = fmaf(q4[e], S[e0 + e], o4[e]);
-        if (MODE == 1 && KIND == 0) decp[e0 + e] *= a4[e];
+        if (MODE == 1 && KIND != 1) decp[e0 + e] *= a4[e];
       }
     }
     if (MODE == 1) {
@@ -182,6 +214,14 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
     if (onv) po[c][x] = (o4[0] + o4[1]) + (o4[2] + o4[3]);
     lds_barrier();
     float o = 0.f, ss = 0.f;
+    if (KIND == 2) {
+      if (c == 0 && onv) {
+        for (int g = 0; g < NS; ++g) o += po[g][x];
+        o = fmaf(skip, cv, o);
+        reinterpret_cast<float*>(out)[(size_t)t * H * V + (size_t)hd * V + x] = o * cg / (1.f + expf(-cg));
+      }
+      continue;      // po is next written after the next token's first barrier
+    }
     if (c == 0) {
       if (onv)
         for (int g = 0; g < NS; ++g) o += po[g][x];
@@ -218,7 +258,7 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       if (MODE == 1) dst[(size_t)D * V + D + 1] = fsum;
     }
   }
-  if (KIND == 0 && MODE == 1 && x == 0) {
+  if (KIND != 1 && MODE == 1 && x == 0) {
 #pragma unroll
     for (int e = 0; e < CH; ++e)
       if (i0 + e < D) dst[(size_t)D * V + i0 + e] = decp[e];
@@ -295,9 +335,11 @@ extern "C" long long k8s_gated_scan_workspace(int T, int nseq, int H, int D, int
 extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, int cq, int ck, int cv, int ci, int cf,
                               int cg, const void* fbias, const void* ibias, const void* lower, const void* normw,
                               float* state, const int* cu_q, const int* seq_slots, const int* positions, int nseq, int H,
-                              int D, int V, float eps, float cap, int f32, int T, int Lc, float* ws, hipStream_t s) {
+                              int D, int V, float eps, float cap, int f32, int T, int Lc, float* ws, const float* aux,
+                              long ldaux, const float* hpar, int R, hipStream_t s) {
   if (nseq <= 0) return 0;
-  if (H <= 0 || H > 65535 || D <= 0 || D > 256 || V <= 0 || V > 256 || kind < 0 || kind > 1) return -1;
+  if (H <= 0 || H > 65535 || D <= 0 || D > 256 || V <= 0 || V > 256 || kind < 0 || kind > 2) return -1;
+  if (kind == 2 && (aux == nullptr || hpar == nullptr || R <= 0 || H % R)) return -1;
   if (kind == 0 && lower == nullptr) return -1;
   if (kind == 1 && !(cap > 0.f)) return -1;
   const int m = D > V ? D : V, DX = (m + 63) / 64 * 64;
@@ -309,17 +351,18 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
 #define K8S_GS(TA, CH, KIND, MODE, GX, LOC, START)                                                                  \
   gated_scan_kernel<TA, CH, KIND, MODE><<<dim3(GX, H), block, 0, s>>>(                                              \
       (TA*)out, proj, ld, co, (const TA*)fbias, (const TA*)ibias, (const TA*)lower, (const TA*)normw, state, cu_q,  \
-      seq_slots, positions, H, D, V, eps, cap, nseq, Lc, LOC, START)
+      seq_slots, positions, H, D, V, eps, cap, nseq, Lc, LOC, START, aux, ldaux, hpar, R)
 #define K8S_GS_C(TA, KIND, MODE, GX, LOC, START)                     \
   do {                                                               \
     if (ch == 16) K8S_GS(TA, 16, KIND, MODE, GX, LOC, START);        \
     else if (ch == 32) K8S_GS(TA, 32, KIND, MODE, GX, LOC, START);   \
     else K8S_GS(TA, 64, KIND, MODE, GX, LOC, START);                 \
   } while (0)
-#define K8S_GS_K(TA, MODE, GX, LOC, START)                  \
-  do {                                                      \
-    if (kind == 0) K8S_GS_C(TA, 0, MODE, GX, LOC, START);   \
-    else K8S_GS_C(TA, 1, MODE, GX, LOC, START);             \
+#define K8S_GS_K(TA, MODE, GX, LOC, START)                       \
+  do {                                                           \
+    if (kind == 0) K8S_GS_C(TA, 0, MODE, GX, LOC, START);        \
+    else if (kind == 1) K8S_GS_C(TA, 1, MODE, GX, LOC, START);   \
+    else K8S_GS_C(float, 2, MODE, GX, LOC, START);               \
   } while (0)
 #define K8S_GS_T(MODE, GX, LOC, START)                      \
   do {                                                      \
@@ -334,7 +377,7 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
   float* loc = ws;
   float* start = ws + (size_t)chunks * H * ((size_t)D * V + D + 2);
   K8S_GS_T(1, chunks, loc, nullptr);
-  if (kind == 0)
+  if (kind != 1)     // one decay per key channel (KIND 2: the head's, repeated)
     gated_prefix_kernel<0><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
   else
     gated_prefix_kernel<1><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);

@@ -220,21 +220,23 @@ __global__ void wkv_prefix_kernel(float* __restrict__ cs_start, const float* __r
 
 // One workgroup per token: cache[slot] = [rms(dkv[:C]) * normw | rope(dkv[C:])] and the rotated part of every
 // head of q ([T, H, Dn + R], last R of a head) rotated in place.  Rotation pairs dimension i with i + dims / 2 over
-// the first `dims` rotated dimensions; cos_sin[pos] = [cos(dims / 2) | sin(dims / 2)].
+// the first `dims` rotated dimensions (`interleaved`: dimension 2i with 2i + 1); cos_sin[pos] = [cos(dims / 2) |
+// sin(dims / 2)].  `ldd`: the row stride of dkv (a view into a wider projection).
 template <typename TA>
 __global__ __launch_bounds__(256) void latent_kv_write_kernel(TA* __restrict__ cache, const TA* __restrict__ dkv,
                                                               const TA* __restrict__ normw, TA* __restrict__ q,
                                                               const float* __restrict__ cos_sin,
                                                               const int* __restrict__ positions,
                                                               const int* __restrict__ slot_mapping, int C, int R, int H,
-                                                              int Dn, int dims, float eps) {
+                                                              int Dn, int dims, float eps, long ldd, int interleaved) {
   __shared__ float red[16];
   const int t = blockIdx.x;
   const int pos = positions[t];
   if (pos < 0) return;
   const int slot = slot_mapping[t];
   const int L = C + R, half = dims / 2;
-  const TA* d = dkv + (size_t)t * L;
+  const TA* d = dkv + (size_t)t * ldd;
+  const int ia = interleaved ? 2 : 1, ib = interleaved ? 1 : half;   // pair i = elements (ia i, ia i + ib)
   float ss = 0.f;
   for (int i = threadIdx.x; i < C; i += blockDim.x) {
     const float x = ldf(d, i);
@@ -247,9 +249,10 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(TA* __restrict__ c
     TA* row = cache + (size_t)slot * L;
     for (int i = threadIdx.x; i < C; i += blockDim.x) stf(row, i, ldf(d, i) * inv * ldf(normw, i));
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      const float a = ldf(d, C + i), b = ldf(d, C + half + i), c = cs[i], sn = cs[half + i];
-      stf(row, C + i, a * c - b * sn);
-      stf(row, C + half + i, b * c + a * sn);
+      const int e0 = C + ia * i, e1 = e0 + ib;
+      const float a = ldf(d, e0), b = ldf(d, e1), c = cs[i], sn = cs[half + i];
+      stf(row, e0, a * c - b * sn);
+      stf(row, e1, b * c + a * sn);
     }
     for (int i = dims + threadIdx.x; i < R; i += blockDim.x) stf(row, C + i, ldf(d, C + i));
   }
@@ -257,22 +260,24 @@ __global__ __launch_bounds__(256) void latent_kv_write_kernel(TA* __restrict__ c
   for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
     const int hh = idx / half, i = idx - hh * half;
     TA* qh = qt + (size_t)hh * (Dn + R) + Dn;
-    const float a = ldf(qh, i), b = ldf(qh, half + i), c = cs[i], sn = cs[half + i];
-    stf(qh, i, a * c - b * sn);
-    stf(qh, half + i, b * c + a * sn);
+    const int e0 = ia * i, e1 = e0 + ib;
+    const float a = ldf(qh, e0), b = ldf(qh, e1), c = cs[i], sn = cs[half + i];
+    stf(qh, e0, a * c - b * sn);
+    stf(qh, e1, b * c + a * sn);
   }
 }
 
 // One workgroup per token, one wave per head (heads beyond the wave count take further passes).  Keys come in blocks
 // of KB <= 64 cached rows staged in LDS as fp32 and shared by the heads; lane l scores key l of the block
 // ((q_abs . c + q_rot . k_rot) * scale), the block joins a running softmax, and lane l accumulates latent
-// dimensions l, l + 64, ... of sum_j p_j c_j.  out [T, H, C] = that sum / the softmax denominator.
+// dimensions l, l + 64, ... of sum_j p_j c_j.  out [T, H, C] = that sum / the softmax denominator.  `sinks` [H] fp32
+// (optional): the denominator of head h holds one more term e^sinks[h], which has no key and no value.
 template <typename TA, int NACC>
 __global__ void latent_attention_kernel(TA* __restrict__ out, const TA* __restrict__ q_abs, const TA* __restrict__ q,
                                         const TA* __restrict__ cache, const int* __restrict__ block_tables,
                                         int max_blocks, const int* __restrict__ tok_seq,
                                         const int* __restrict__ positions, int C, int R, int H, int Dn, int window,
-                                        float scale, int bs, int KB) {
+                                        float scale, int bs, int KB, const float* __restrict__ sinks) {
   extern __shared__ float smem[];
   const int t = blockIdx.x;
   const int p = positions[t];
@@ -333,10 +338,15 @@ __global__ void latent_attention_kernel(TA* __restrict__ out, const TA* __restri
       }
     }
     if (hv) {
+      float inv = 1.f / l;
+      if (sinks != nullptr) {          // join the sink under a common maximum
+        const float sk = sinks[hd], mx = fmaxf(m, sk), am = expf(m - mx);
+        inv = am / (l * am + expf(sk - mx));
+      }
 #pragma unroll
       for (int i = 0; i < NACC; ++i) {
         const int d = lane + 64 * i;
-        if (d < C) stf(out, ((size_t)t * H + hd) * C + d, acc[i] / l);
+        if (d < C) stf(out, ((size_t)t * H + hd) * C + d, acc[i] * inv);
       }
     }
   }
@@ -360,7 +370,7 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ pacc, float* __restrict__ pml, const bf16_t* __restrict__ q_abs,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ cu_q, int C, int R,
-    int H, int Dn, int window, float scale, int bs, int nsplit) {
+    int H, int Dn, int window, float scale, int bs, int nsplit, const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) char smem_b[];
   char* klds = smem_b;               // [32][L + 8] bf16
   const int hg = blockIdx.y;
@@ -517,7 +527,11 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     const int hd = hg * 16 + 4 * g + i;
     if (hd >= H) continue;
     if (nsplit == 1) {
-      const float inv = 1.f / l_i[i];
+      float inv = 1.f / l_i[i];
+      if (sinks != nullptr) {
+        const float sk = sinks[hd], mx = fmaxf(m_i[i], sk), am = expf(m_i[i] - mx);
+        inv = am / (l_i[i] * am + expf(sk - mx));
+      }
 #pragma unroll
       for (int n = 0; n < NDB; ++n)
         if (n < ndb) out[((size_t)t * H + hd) * C + 16 * n + li] = f2bf(o[n][i] * inv);
@@ -537,16 +551,16 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
 // out[t][head] = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the key splits
 __global__ void latent_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ pacc,
                                     const float* __restrict__ pml, const int* __restrict__ positions, int C, int H,
-                                    int HP, int nsplit) {
+                                    int HP, int nsplit, const float* __restrict__ sinks) {
   const int t = blockIdx.x, hd = blockIdx.y;
   if (positions[t] < 0) {
     for (int d = threadIdx.x; d < C; d += blockDim.x) out[((size_t)t * H + hd) * C + d] = 0;
     return;
   }
   const size_t rec0 = ((size_t)t * HP + hd) * nsplit;
-  float M = -INFINITY;
+  float M = sinks != nullptr ? sinks[hd] : -INFINITY;
   for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pml[(rec0 + s) * 2]);
-  float den = 0.f;
+  float den = sinks != nullptr ? expf(sinks[hd] - M) : 0.f;
   for (int s = 0; s < nsplit; ++s) {
     const float ms = pml[(rec0 + s) * 2];
     if (ms != -INFINITY) den += expf(ms - M) * pml[(rec0 + s) * 2 + 1];
@@ -630,23 +644,24 @@ extern "C" int k8s_wkv_scan(void* out, const void* r, const void* k, const void*
 
 extern "C" int k8s_latent_kv_write(void* cache, const void* dkv, const void* normw, void* q, const float* cos_sin,
                                    const int* positions, const int* slot_mapping, int T, int C, int R, int H, int Dn,
-                                   int dims, float eps, int f32, hipStream_t s) {
+                                   int dims, float eps, int f32, long ldd, int interleaved, hipStream_t s) {
   if (T <= 0) return 0;
-  if (C <= 0 || R < 0 || dims < 0 || dims > R || (dims & 1) || H <= 0) return -1;
+  if (C <= 0 || R < 0 || dims < 0 || dims > R || (dims & 1) || H <= 0 || ldd < C + R) return -1;
   if (f32)
     latent_kv_write_kernel<float><<<T, 256, 0, s>>>((float*)cache, (const float*)dkv, (const float*)normw, (float*)q,
-                                                    cos_sin, positions, slot_mapping, C, R, H, Dn, dims, eps);
+                                                    cos_sin, positions, slot_mapping, C, R, H, Dn, dims, eps, ldd,
+                                                    interleaved);
   else
     latent_kv_write_kernel<bf16_t><<<T, 256, 0, s>>>((bf16_t*)cache, (const bf16_t*)dkv, (const bf16_t*)normw,
                                                      (bf16_t*)q, cos_sin, positions, slot_mapping, C, R, H, Dn, dims,
-                                                     eps);
+                                                     eps, ldd, interleaved);
   return (int)hipGetLastError();
 }
 
 extern "C" int k8s_latent_attention(void* out, const void* q_abs, const void* q, const void* cache,
                                     const int* block_tables, int max_blocks, const int* tok_seq, const int* positions,
                                     int T, int C, int R, int H, int Dn, int window, float scale, int bs, int f32,
-                                    hipStream_t s) {
+                                    const float* sinks, hipStream_t s) {
   if (T <= 0) return 0;
   if (C <= 0 || C > 512 || R < 0 || H <= 0 || bs <= 0) return -1;
   const int L = C + R;
@@ -660,7 +675,7 @@ extern "C" int k8s_latent_attention(void* out, const void* q_abs, const void* q,
 #define K8S_LA(TA, NA) \
   latent_attention_kernel<TA, NA><<<T, nw * 64, lds, s>>>((TA*)out, (const TA*)q_abs, (const TA*)q, (const TA*)cache, \
                                                           block_tables, max_blocks, tok_seq, positions, C, R, H, Dn, \
-                                                          window, scale, bs, KB)
+                                                          window, scale, bs, KB, sinks)
 #define K8S_LA_T(TA)                  \
   do {                                \
     if (nacc <= 1) K8S_LA(TA, 1);     \
@@ -687,7 +702,7 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
                                          const void* cache, const int* block_tables, int max_blocks,
                                          const int* tok_seq, const int* positions, int T, int C, int R, int H, int Dn,
                                          int window, float scale, int bs, int nsplit, const int* cu_q, int nseq,
-                                         int max_qlen, hipStream_t s) {
+                                         int max_qlen, const float* sinks, hipStream_t s) {
   if (T <= 0) return 0;
   if (!k8s_latent_mfma_ok(C, R, Dn) || H <= 0 || bs <= 0 || nsplit < 1 || (nsplit > 1 && (!pacc || !pml))) return -1;
   const int L = C + R, HG = (H + 15) / 16;
@@ -700,11 +715,11 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
     if (tiles)                                                                                                        \
       latent_attention_mfma_kernel<NDB, NKK, 4><<<grid, 256, lds, s>>>(                                               \
           (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
-          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit);                              \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks);                       \
     else                                                                                                              \
       latent_attention_mfma_kernel<NDB, NKK, 1><<<grid, 64, lds, s>>>(                                                \
           (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
-          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit);                              \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks);                       \
   } while (0)
   if (C <= 128 && L <= 256) K8S_LM(8, 8);
   else if (C <= 256 && L <= 256) K8S_LM(16, 8);
@@ -712,6 +727,7 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
   else K8S_LM(32, 20);
 #undef K8S_LM
   if (nsplit > 1)
-    latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit);
+    latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit,
+                                                   sinks);
   return (int)hipGetLastError();
 }

@@ -59,6 +59,49 @@ __global__ __launch_bounds__(256) void resnorm_kernel(float* __restrict__ x, con
   }
 }
 
+// Norm after the sum: x[t] <- (alpha x[t] + c1 branch[t] + c2 branch2[t]) / sqrt(mean(.^2) + eps) * gain, stored back
+// in fp32 (the stream stays normed); `out` (optional) receives the same row in the activation type, for the sublayer
+// that reads it next.  `gain` is one number for the whole row.  One workgroup per row; the row is held in registers
+// (W <= 256 * 16) or re-formed from its inputs on the second pass.
+template <typename TA>
+__global__ __launch_bounds__(256) void postnorm_kernel(float* __restrict__ x, const TA* __restrict__ branch,
+                                                       const TA* __restrict__ branch2, float alpha, float c1, float c2,
+                                                       float gain, float eps, TA* __restrict__ out, int W) {
+  __shared__ float red[16];
+  const size_t base = (size_t)blockIdx.x * W;
+  auto value = [&](int i) -> float {
+    float v = alpha * x[base + i];
+    if (branch != nullptr) v = fmaf(c1, ldf(branch, base + i), v);
+    if (branch2 != nullptr) v = fmaf(c2, ldf(branch2, base + i), v);
+    return v;
+  };
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float v = value(i);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float m = gain / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float y = value(i) * m;      // element i is read and written by this thread only
+    x[base + i] = y;
+    if (out != nullptr) stf(out, base + i, y);
+  }
+}
+
+// out[t, c] = y[t, c] * f(gate[t, c]) with f = sigmoid (kind 0) or silu (kind 1); y and gate are row-strided views.
+template <typename TY, typename TA>
+__global__ void gate_mul_kernel(TA* __restrict__ out, const TY* __restrict__ y, long ldy, const TA* __restrict__ gate,
+                                long ldg, int T, int F, int kind) {
+  const size_t n = (size_t)T * F;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = i / F, c = i - t * F;
+    const float g = ldf(gate, t * ldg + c);
+    const float s = 1.f / (1.f + expf(-g));
+    stf(out, i, ldf(y, t * ldy + c) * (kind == 1 ? g * s : s));
+  }
+}
+
 // kinds: 0 gelu_tanh(g) * u, 1 g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit)
 // (limit <= 0: no clamp), 5 relu(g) * u -- these read [T, 2F] = [gate | up]; 2 tanh, 3 silu, 4 erf-gelu,
 // 6 limit * tanh(x / limit): elementwise on [T, F].
@@ -99,16 +142,35 @@ __global__ void act_kernel(TA* __restrict__ out, const TA* __restrict__ x, int T
 }
 
 // out[t] = ca * a[t] / rms(a[t]) * wa + cb * b[t] / rms(b[t]) * wb (b optional): the outputs of two mixers that run side
-// by side, each normed over the row in fp32, joined.  One workgroup per row.
+// by side, each normed over the row in fp32, joined.  One workgroup per row.  `lda`: the row stride of a (a view into a
+// wider projection).  groups > 1 (a alone): every one of that many equal consecutive parts of the row is divided by its
+// own root mean square, one wave per part.
 template <typename TA, typename TO>
-__global__ __launch_bounds__(256) void norm_mix_kernel(TO* __restrict__ out, const TA* __restrict__ a,
+__global__ __launch_bounds__(256) void norm_mix_kernel(TO* __restrict__ out, const TA* __restrict__ a, long lda,
                                                        const TA* __restrict__ wa, const TA* __restrict__ b,
-                                                       const TA* __restrict__ wb, float eps, float ca, float cb, int W) {
+                                                       const TA* __restrict__ wb, float eps, float ca, float cb, int W,
+                                                       int groups) {
   __shared__ float red[16];
   const size_t base = (size_t)blockIdx.x * W;
+  const TA* ar = a + (size_t)blockIdx.x * lda;
+  if (groups > 1) {
+    const int Wg = W / groups, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    for (int g = wave; g < groups; g += nw) {
+      const size_t o = (size_t)g * Wg;
+      float sg = 0.f;
+      for (int i = lane; i < Wg; i += 64) {
+        const float v = ldf(ar, o + i);
+        sg += v * v;
+      }
+      sg = wave_sum(sg);
+      const float inv = ca / sqrtf(sg / (float)Wg + eps);
+      for (int i = lane; i < Wg; i += 64) stf(out, base + o + i, ldf(ar, o + i) * inv * ldf(wa, o + i));
+    }
+    return;
+  }
   float sa = 0.f, sb = 0.f;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    const float va = ldf(a, base + i);
+    const float va = ldf(ar, i);
     sa += va * va;
     if (b != nullptr) {
       const float vb = ldf(b, base + i);
@@ -123,7 +185,7 @@ __global__ __launch_bounds__(256) void norm_mix_kernel(TO* __restrict__ out, con
     ib = cb / sqrtf(sb / (float)W + eps);
   }
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float y = ldf(a, base + i) * ia * ldf(wa, i);
+    float y = ldf(ar, i) * ia * ldf(wa, i);
     if (b != nullptr) y += ldf(b, base + i) * ib * ldf(wb, i);
     stf(out, base + i, y);
   }
@@ -328,18 +390,52 @@ extern "C" int k8s_resnorm(float* x, const void* branch, const void* branch2, fl
   return (int)hipGetLastError();
 }
 
-extern "C" int k8s_norm_mix(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, float ca,
-                            float cb, int T, int W, int in_f32, int out_f32, hipStream_t s) {
+extern "C" int k8s_norm_mix(void* out, const void* a, long lda, const void* wa, const void* b, const void* wb,
+                            float eps, float ca, float cb, int T, int W, int groups, int in_f32, int out_f32,
+                            hipStream_t s) {
   if (T <= 0) return 0;
-  if (W <= 0 || a == nullptr || wa == nullptr || (b != nullptr && wb == nullptr)) return -1;
-#define K8S_NM(TA, TO)                                                                                              \
-  norm_mix_kernel<TA, TO><<<T, 256, 0, s>>>((TO*)out, (const TA*)a, (const TA*)wa, (const TA*)b, (const TA*)wb, eps, \
-                                            ca, cb, W)
+  if (W <= 0 || a == nullptr || wa == nullptr || (b != nullptr && wb == nullptr) || lda < W) return -1;
+  if (groups < 1 || W % groups || (groups > 1 && b != nullptr)) return -1;
+#define K8S_NM(TA, TO)                                                                                             \
+  norm_mix_kernel<TA, TO><<<T, 256, 0, s>>>((TO*)out, (const TA*)a, lda, (const TA*)wa, (const TA*)b, (const TA*)wb, \
+                                            eps, ca, cb, W, groups)
   if (in_f32 && out_f32) K8S_NM(float, float);
   else if (in_f32) K8S_NM(float, bf16_t);
   else if (out_f32) K8S_NM(bf16_t, float);
   else K8S_NM(bf16_t, bf16_t);
 #undef K8S_NM
+  return (int)hipGetLastError();
+}
+
+extern "C" int k8s_postnorm(float* x, const void* branch, const void* branch2, float alpha, float c1, float c2,
+                            float gain, float eps, void* out, int T, int W, int f32, hipStream_t s) {
+  if (T <= 0) return 0;
+  if (W <= 0 || x == nullptr || (branch2 != nullptr && branch == nullptr)) return -1;
+  if (f32)
+    postnorm_kernel<float><<<T, 256, 0, s>>>(x, (const float*)branch, (const float*)branch2, alpha, c1, c2, gain, eps,
+                                             (float*)out, W);
+  else
+    postnorm_kernel<bf16_t><<<T, 256, 0, s>>>(x, (const bf16_t*)branch, (const bf16_t*)branch2, alpha, c1, c2, gain,
+                                              eps, (bf16_t*)out, W);
+  return (int)hipGetLastError();
+}
+
+// y_f32: y is fp32 whatever the activation type (an fp32 intermediate gated into the activation type)
+extern "C" int k8s_gate_mul(void* out, const void* y, long ldy, const void* gate, long ldg, int T, int F, int kind,
+                            int y_f32, int f32, hipStream_t s) {
+  if (T <= 0 || F <= 0) return 0;
+  if (kind < 0 || kind > 1 || ldy < F || ldg < F || (f32 && !y_f32)) return -1;
+  const size_t n = (size_t)T * F;
+  const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
+  if (f32)
+    gate_mul_kernel<float, float><<<blocks, 256, 0, s>>>((float*)out, (const float*)y, ldy, (const float*)gate, ldg, T,
+                                                         F, kind);
+  else if (y_f32)
+    gate_mul_kernel<float, bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, (const float*)y, ldy, (const bf16_t*)gate, ldg,
+                                                          T, F, kind);
+  else
+    gate_mul_kernel<bf16_t, bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)y, ldy, (const bf16_t*)gate,
+                                                           ldg, T, F, kind);
   return (int)hipGetLastError();
 }
 

@@ -25,7 +25,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 // One workgroup per token, one wave per head vector (H query heads, then G key heads; further passes when there are
 // more vectors than waves).  x = proj + bias; (qnw / knw) x = x / rms(whole q or k projection) * weight;
 // (x[2i], x[2i + 1]) -- half layout: (x[i], x[i + dims / 2]) -- turns by the angle of cos_sin[pos] = [cos(dims / 2) |
-// sin(dims / 2)]; then x / sqrt(mean(x^2) + eps) when `unit`.  Queries are written back in place, keys to
+// sin(dims / 2)]; then x / sqrt(mean(x^2) + eps) when `unit`.  (hqw / hkw [D]) before the rotation every head is
+// divided by its own root mean square and multiplied by the weight, the same for all heads.  Queries are written back
+// in place, keys to
 // kcache[slot][g][D].  Values: v = proj + bias, then (vfirst_in) v = (1 - lam) v + lam vfirst_in[t]; (vfirst_out)
 // vfirst_out[t] = v in fp32; vcache[slot][g][V] = v.
 template <typename TA>
@@ -34,7 +36,8 @@ __global__ __launch_bounds__(256) void window_kv_write_kernel(
     const TA* __restrict__ qb, const TA* __restrict__ kb, const TA* __restrict__ vb, const float* __restrict__ cos_sin,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping, const float* __restrict__ vfirst_in,
     float* __restrict__ vfirst_out, float lam, int H, int G, int D, int V, int dims, float eps, int unit,
-    int half_layout, const TA* __restrict__ qnw, const TA* __restrict__ knw) {
+    int half_layout, const TA* __restrict__ qnw, const TA* __restrict__ knw, const TA* __restrict__ hqw,
+    const TA* __restrict__ hkw) {
   extern __shared__ float xs[];   // [waves][D]
   __shared__ float red[16];
   const int t = blockIdx.x;
@@ -69,11 +72,18 @@ __global__ __launch_bounds__(256) void window_kv_write_kernel(
     const TA* src = row + (isq ? 0 : koff) + (size_t)hd * D;
     const TA* bias = isq ? qb : kb;
     const TA* nrm = isq ? qnw : knw;
+    const TA* hnw = isq ? hqw : hkw;
     const float inv0 = isq ? invq : invk;
+    float hs = 0.f;
     for (int d = lane; d < D; d += 64) {
       float v = ldf(src, d) + (bias != nullptr ? ldf(bias, (size_t)hd * D + d) : 0.f);
       if (nrm != nullptr) v *= inv0 * ldf(nrm, (size_t)hd * D + d);
       x[d] = v;
+      hs += v * v;
+    }
+    if (hnw != nullptr) {            // uniform over the wave; every lane rescales the elements it wrote itself
+      const float hinv = 1.0f / sqrtf(wave_sum(hs) / (float)D + eps);
+      for (int d = lane; d < D; d += 64) x[d] *= hinv * ldf(hnw, d);
     }
     wave_lds_sync();
     float ss = 0.f;
@@ -651,7 +661,8 @@ extern "C" int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long l
                                    const void* kb, const void* vb, const float* cos_sin, const int* positions,
                                    const int* slot_mapping, const float* vfirst_in, float* vfirst_out, float lam, int T,
                                    int H, int G, int D, int V, int dims, float eps, int unit, int half_layout,
-                                   const void* qnw, const void* knw, int f32, hipStream_t s) {
+                                   const void* qnw, const void* knw, const void* hqw, const void* hkw, int f32,
+                                   hipStream_t s) {
   if (T <= 0) return 0;
   // G == 0: a layer that attends another layer's cache prepares its queries only
   if (H <= 0 || G < 0 || (G > 0 && H % G) || D <= 0 || D > 512 || V <= 0 || dims < 0 || dims > D || (dims & 1)) return -1;
@@ -662,7 +673,7 @@ extern "C" int k8s_window_kv_write(void* kcache, void* vcache, void* qkv, long l
   window_kv_write_kernel<TA><<<T, 256, lds, s>>>((TA*)kcache, (TA*)vcache, (TA*)qkv, ld, koff, voff, (const TA*)qb,    \
                                                  (const TA*)kb, (const TA*)vb, cos_sin, positions, slot_mapping,      \
                                                  vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit, half_layout, \
-                                                 (const TA*)qnw, (const TA*)knw)
+                                                 (const TA*)qnw, (const TA*)knw, (const TA*)hqw, (const TA*)hkw)
   if (f32) K8S_WKW(float);
   else K8S_WKW(bf16_t);
 #undef K8S_WKW

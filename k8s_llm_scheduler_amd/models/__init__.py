@@ -15,10 +15,10 @@ def _architecture(c: dict) -> str:
 
 def load_config(name_or_path: str):
     """The configuration object of a preset or checkpoint."""
-    from . import nukizen, putulorn, rupatar
+    from . import nukizen, putulorn, rupatar, semanex
     from .config import get_config
 
-    designs = (putulorn, rupatar, nukizen)
+    designs = (putulorn, rupatar, nukizen, semanex)
     for d in designs:
         if name_or_path in d.PRESETS:
             return d.PRESETS[name_or_path]
@@ -40,6 +40,7 @@ def model_class(cfg):
     from .nukizen import NukizenConfig, NukizenModel
     from .putulorn import PutulornConfig, PutulornModel
     from .rupatar import RupatarConfig, RupatarModel
+    from .semanex import SemanexConfig, SemanexModel
 
     if isinstance(cfg, PutulornConfig):
         return PutulornModel
@@ -47,6 +48,8 @@ def model_class(cfg):
         return RupatarModel
     if isinstance(cfg, NukizenConfig):
         return NukizenModel
+    if isinstance(cfg, SemanexConfig):
+        return SemanexModel
     if isinstance(cfg, LlamaConfig):
         return LlamaModel
     raise TypeError(f"no model class for {type(cfg).__name__}")

@@ -523,6 +523,30 @@ def resnorm(x: torch.Tensor, branch, mult: float, rowvec, w, offset: float, eps:
     return y.to(out_dtype)
 
 
+def postnorm(x: torch.Tensor, branch, branch2, alpha: float, c1: float, c2: float, gain: float, eps: float, out_dtype):
+    """x (fp32, in place) <- v / sqrt(mean(v^2) + eps) * gain with v = alpha x + c1 branch + c2 branch2; returns the new
+    rows in ``out_dtype`` (None: nothing)."""
+    v = alpha * x
+    if branch is not None:
+        v = v + c1 * branch.float()
+    if branch2 is not None:
+        v = v + c2 * branch2.float()
+    x.copy_(v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * gain)
+    return x.to(out_dtype) if out_dtype is not None else None
+
+
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def gate_mul(y: torch.Tensor, gate: torch.Tensor, kind: int) -> torch.Tensor:
+    """y * sigmoid(gate), or y * silu(gate), in the gate's type."""
+    g = gate.float()
+    f = torch.sigmoid(g)
+    if kind == GATE_SILU:
+        f = f * g
+    return (y.float() * f).to(gate.dtype)
+
+
 def act(x: torch.Tensor, kind: int, limit: float = 0.0, alpha: float = 1.0, row_scale=None, row_map=None) -> torch.Tensor:
     """Gated kinds (ACT_GELU_TANH, ACT_SWISH_CLAMP, ACT_RELU: relu(g) u) take [T, 2F] = [gate | up] and return [T, F];
     ACT_TANH / ACT_SILU / ACT_GELU_ERF / ACT_SOFTCAP (limit tanh(x / limit)) are elementwise and take a factor per row:
@@ -627,9 +651,10 @@ def wkv_scan(r, k, v, g, z, w0, u, lnw, state, cu_q, seq_slots, positions, H: in
 
 # ----------------------------------------------------------------------------- latent attention
 def latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C: int, R: int, H: int, Dn: int,
-                    rot_dims: int, eps: float) -> None:
+                    rot_dims: int, eps: float, interleaved: bool = False) -> None:
     """cache[slot] = [rms(dkv[:C]) * normw | rope(dkv[C:])]; q's rotated part ([T, H, Dn + R], last R of each head)
-    is rotated in place.  Rows with a negative slot are not written."""
+    is rotated in place (pairs (i, i + rot_dims / 2), or (2i, 2i + 1) when ``interleaved``).  Rows with a negative
+    slot are not written."""
     T = dkv.shape[0]
     d = dkv.float()
     c = d[:, :C] * torch.rsqrt(d[:, :C].pow(2).mean(-1, keepdim=True) + eps) * normw.float()
@@ -638,6 +663,11 @@ def latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C: i
     cos, sin = cs[:, :half], cs[:, half:]
 
     def rot(x, cos, sin):
+        if interleaved:
+            y = x.clone()
+            a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+            y[..., 0:rot_dims:2], y[..., 1:rot_dims:2] = a * cos - b * sin, b * cos + a * sin
+            return y
         a, b = x[..., :half], x[..., half:rot_dims]
         return torch.cat([a * cos - b * sin, b * cos + a * sin, x[..., rot_dims:]], -1)
 
@@ -650,9 +680,10 @@ def latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C: i
 
 
 def latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C: int, R: int, H: int, Dn: int,
-                     window: int, scale: float, block_size: int, out_dtype):
+                     window: int, scale: float, block_size: int, out_dtype, sinks=None):
     """Token t of sequence tok_seq[t] at position p attends the cached rows of positions max(0, p - window + 1) .. p
-    (window <= 0: all): score = (q_abs . c + q_rot . k_rot) * scale, softmax, returns sum p c  [T, H, C]."""
+    (window <= 0: all): score = (q_abs . c + q_rot . k_rot) * scale, softmax (``sinks`` [H]: one more term e^sinks[h]
+    in head h's denominator), returns sum p c  [T, H, C]."""
     T = q_abs.shape[0]
     out = torch.zeros(T, H, C)
     qa = q_abs.float().view(T, H, C)
@@ -666,6 +697,11 @@ def latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C: int, 
         bt = block_tables[int(tok_seq[t])].long()
         rows = cache[bt[js // block_size] * block_size + js % block_size].float()
         s = (qa[t] @ rows[:, :C].T + qr[t] @ rows[:, C:].T) * scale
+        if sinks is not None:
+            mx = torch.maximum(s.max(-1, keepdim=True).values, sinks.float().view(H, 1))
+            e = torch.exp(s - mx)
+            out[t] = (e / (e.sum(-1, keepdim=True) + torch.exp(sinks.float().view(H, 1) - mx))) @ rows[:, :C]
+            continue
         out[t] = torch.softmax(s, -1) @ rows[:, :C]
     return out.to(out_dtype)
 
@@ -727,11 +763,12 @@ def pool_entry(bt_row, b: int, P: int, bs: int) -> int:
 
 def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_sin, positions, slot_mapping, vfirst_in,
                     vfirst_out, lam: float, H: int, G: int, D: int, V: int, dims: int, eps: float, unit: bool,
-                    half_layout: bool = False, qnw=None, knw=None) -> None:
+                    half_layout: bool = False, qnw=None, knw=None, head_qnw=None, head_knw=None) -> None:
     """Per token: q (first H D columns of qkv, rewritten in place) and k (at koff) get their bias, (``qnw`` / ``knw``)
     the RMS norm over the whole projection (all heads at once) with that weight, the rotation of the pairs
     (2i, 2i + 1) -- ``half_layout``: (i, i + dims / 2) --, i < dims / 2, by cos_sin[pos] = [cos | sin], and (``unit``)
-    x / sqrt(mean(x^2) + eps) per head; v (at voff) gets its bias and (``vfirst_in``) becomes (1 - lam) v + lam
+    x / sqrt(mean(x^2) + eps) per head; ``head_qnw`` / ``head_knw`` [D]: before the rotation every head is divided by
+    its own root mean square and multiplied by that weight; v (at voff) gets its bias and (``vfirst_in``) becomes (1 - lam) v + lam
     vfirst_in; ``vfirst_out`` receives v in fp32.  k, v go to kcache [slots, G, D] / vcache [slots, G, V] at the tokens'
     slots (negative: not written); ``kcache`` None: queries only.  Rows with a negative position are skipped."""
     T = qkv.shape[0]
@@ -739,12 +776,14 @@ def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_s
     half = dims // 2
     cs = cos_sin[positions.long().clamp(min=0)] if dims else None
 
-    def prep(x, bias, n, nw):
-        x = x.float().view(T, n, D)
+    def prep(x, bias, n, nw, hnw):
+        x = x.float().reshape(T, n, D)
         if bias is not None:
             x = x + bias.float().view(n, D)
         if nw is not None:
             x = x * torch.rsqrt(x.pow(2).mean((-2, -1), keepdim=True) + eps) * nw.float().view(n, D)
+        if hnw is not None:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * hnw.float().view(D)
         if dims:
             c, s = cs[:, None, :half], cs[:, None, half:]
             x = x.clone()
@@ -758,11 +797,11 @@ def window_kv_write(kcache, vcache, qkv, koff: int, voff: int, qb, kb, vb, cos_s
             x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
         return x
 
-    q = prep(qkv[:, :H * D], qb, H, qnw).reshape(T, H * D)
+    q = prep(qkv[:, :H * D], qb, H, qnw, head_qnw).reshape(T, H * D)
     qkv[live, :H * D] = q[live].to(qkv.dtype)
     if kcache is None:
         return
-    k = prep(qkv[:, koff:koff + G * D], kb, G, knw)
+    k = prep(qkv[:, koff:koff + G * D], kb, G, knw, head_knw)
     v = qkv[:, voff:voff + G * V].float()
     if vb is not None:
         v = v + vb.float()
@@ -836,20 +875,51 @@ def window_attention(q, gate, kcache, vcache, kpool, vpool, block_tables, tok_se
 
 
 # ----------------------------------------------------------------------------- gated matrix-state recurrences
-SCAN_HGRN2, SCAN_MLSTM = 0, 1
+SCAN_HGRN2, SCAN_MLSTM, SCAN_SSD = 0, 1, 2
 
 
 def gated_scan_record(kind: int, D: int, V: int) -> int:
     return D * V + (D + 1 if kind == SCAN_MLSTM else 0)
 
 
+def ssd_scan(proj, cols: dict, aux, head_params, state, cu_q, seq_slots, positions, H: int, G: int, D: int, V: int):
+    """``proj`` fp32 holds x (H V, at cols v), B and C (G D each, at cols k and q); ``aux`` fp32 holds the step-size
+    logits (H, at cols f) and the gate (H V, at cols g); ``head_params`` [3, H] = neg_a, dt_bias, skip.  Per head h with
+    the B, C of group h // (H / G): dt = softplus(f + dt_bias), S <- exp(neg_a dt) S + dt B x^T (S [D, V]),
+    y = (S^T C + skip x) * silu(g).  fp32 [T, H V]; ``state`` [slots, H, D V] fp32."""
+    T = proj.shape[0]
+    pf, af = proj.float(), aux.float()
+    x = pf[:, cols["v"]:cols["v"] + H * V].view(T, H, V)
+    B = pf[:, cols["k"]:cols["k"] + G * D].view(T, G, D).repeat_interleave(H // G, 1)
+    C = pf[:, cols["q"]:cols["q"] + G * D].view(T, G, D).repeat_interleave(H // G, 1)
+    neg_a, dt_bias, skip = head_params.float()
+    dt = torch.nn.functional.softplus(af[:, cols["f"]:cols["f"] + H] + dt_bias, threshold=1e9)
+    decay = torch.exp(neg_a * dt)
+    gate = af[:, cols["g"]:cols["g"] + H * V]
+    out = torch.zeros(T, H, V)
+    cu = cu_q.tolist()
+    for s in range(len(cu) - 1):
+        a, b = cu[s], cu[s + 1]
+        if b <= a or int(positions[a]) < 0:
+            continue
+        slot = int(seq_slots[s])
+        S = torch.zeros(H, D, V) if int(positions[a]) == 0 else state[slot].view(H, D, V).clone()
+        for t in range(a, b):
+            S = decay[t].view(H, 1, 1) * S + (dt[t].view(H, 1) * B[t]).unsqueeze(2) * x[t].unsqueeze(1)
+            out[t] = torch.einsum("hdv,hd->hv", S, C[t]) + skip.view(H, 1) * x[t]
+        state[slot] = S.reshape(H, D * V)
+    return out.reshape(T, H * V) * gate * torch.sigmoid(gate)
+
+
 def gated_scan(proj, kind: int, cols: dict, fbias, ibias, lower, normw, state, cu_q, seq_slots, positions, H: int,
-               D: int, V: int, eps: float, cap: float, out_dtype):
+               D: int, V: int, eps: float, cap: float, out_dtype, aux=None, head_params=None, groups: int = 0):
     """``proj`` fp32 [T, ld] holds the parts at the column offsets ``cols``; ``state`` [slots, H, record] fp32.
     SCAN_HGRN2: f = low + (1 - low) sigmoid(zf + bf), S <- diag(f) S + (1 - f) v^T, o = S^T silu(zq),
     y = o / rms(o) * normw [V].  SCAN_MLSTM: i = cap tanh((zi + bi) / cap), f = logsigmoid(cap tanh((zf + bf) / cap)),
     m' = max(f + m, i), S <- e^(f + m - m') S + e^(i - m') k v^T, n likewise, o = S^T q / (max(|n . q|, e^(-m')) + 1e-6)
     with q = zq / sqrt(D), y = o / rms(o) * normw [H V] * sigmoid(zg).  A portion at position 0 starts from zero."""
+    if kind == SCAN_SSD:
+        return ssd_scan(proj, cols, aux, head_params, state, cu_q, seq_slots, positions, H, groups, D, V)
     T = proj.shape[0]
     pf = proj.float()
     out = torch.zeros(T, H, V)
@@ -907,7 +977,7 @@ CONV_NONE, CONV_SILU = 0, 1
 
 
 def short_conv(x, w, state, cu_q, seq_slots, positions, in_bias, out_bias, act: int, unit_cols: int, unit_dim: int,
-               scale_cols: int, scale: float, unit_eps: float):
+               scale_cols: int, scale: float, unit_eps: float, residual: bool = False):
     """Causal convolution over time per channel, over a varlen batch.  ``x`` [T, C] (any row stride), ``w`` [C, taps]
     (the last tap is the current token's), inputs x + in_bias, zeros before position 0; the taps - 1 inputs before a
     portion come from ``state`` [slots, taps - 1, C] fp32, which then receives the portion's last ones.  Then out_bias,
@@ -941,6 +1011,13 @@ def short_conv(x, w, state, cu_q, seq_slots, positions, in_bias, out_bias, act: 
         out = out + out_bias.float()
     if act == CONV_SILU:
         out = out * torch.sigmoid(out)
+    if residual:                      # rows of idle sequences stay zero
+        live = torch.zeros(T, dtype=torch.bool)
+        for s in range(len(cu) - 1):
+            if cu[s + 1] > cu[s] and int(positions[cu[s]]) >= 0:
+                live[cu[s]:cu[s + 1]] = True
+        xin = x.float() + (in_bias.float() if in_bias is not None else 0.0)
+        out = torch.where(live[:, None], out + xin, out)
     if unit_cols:
         u = out[:, :unit_cols].reshape(T, unit_cols // unit_dim, unit_dim)
         out[:, :unit_cols] = (u * torch.rsqrt(u.pow(2).sum(-1, keepdim=True) + unit_eps)).reshape(T, unit_cols)
@@ -1016,9 +1093,14 @@ def rglru_scan(u, gates, gate_bias, decay_rate, proj, ycol: int, ybias, state, c
     return (out * y).to(out_dtype)
 
 
-def norm_mix(a, wa, b, wb, eps: float, ca: float, cb: float, out_dtype):
-    """ca * a / rms(a) * wa + cb * b / rms(b) * wb  (rows; ``b`` may be None)."""
+def norm_mix(a, wa, b, wb, eps: float, ca: float, cb: float, out_dtype, groups: int = 1):
+    """ca * a / rms(a) * wa + cb * b / rms(b) * wb  (rows; ``b`` may be None); ``groups`` > 1: the root mean square of
+    each of that many equal consecutive parts of a row by itself."""
     af = a.float()
+    if groups > 1:
+        ag = af.reshape(af.shape[0], groups, -1)
+        y = ca * (ag * torch.rsqrt(ag.pow(2).mean(-1, keepdim=True) + eps)).reshape(af.shape) * wa.float()
+        return y.to(out_dtype)
     y = ca * af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps) * wa.float()
     if b is not None:
         bf = b.float()

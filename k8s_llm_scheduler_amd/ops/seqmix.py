@@ -17,7 +17,8 @@ import torch
 from . import reference as ref
 from .reference import ACT_GELU_ERF, ACT_GELU_TANH, ACT_RELU, ACT_SILU, ACT_SOFTCAP, ACT_SWISH_CLAMP, ACT_TANH  # noqa: F401
 from .reference import CONV_NONE, CONV_SILU  # noqa: F401
-from .reference import SCAN_HGRN2, SCAN_MLSTM  # noqa: F401
+from .reference import GATE_SIGMOID, GATE_SILU  # noqa: F401
+from .reference import SCAN_HGRN2, SCAN_MLSTM, SCAN_SSD  # noqa: F401
 
 BF16, F32, I32 = torch.bfloat16, torch.float32, torch.int32
 GROUP_BM = 64   # row-tile height of the grouped GEMM (gemm_any_kernel's BM)
@@ -93,18 +94,65 @@ def resnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, *, branch: O
 
 
 def norm_mix(a: torch.Tensor, wa: torch.Tensor, b: Optional[torch.Tensor], wb: Optional[torch.Tensor], eps: float,
-             ca: float = 1.0, cb: float = 1.0, out_dtype=None) -> torch.Tensor:
+             ca: float = 1.0, cb: float = 1.0, out_dtype=None, groups: int = 1) -> torch.Tensor:
     """ca * rms-norm(a) * wa + cb * rms-norm(b) * wb over rows [T, W] (norms in fp32; ``b`` None: the first term
-    only): the outputs of two mixers that run side by side, each normed, joined."""
+    only): the outputs of two mixers that run side by side, each normed, joined.  ``a`` may be a column slice of a
+    wider tensor (row stride free).  ``groups`` > 1 (``a`` alone): every one of that many equal consecutive parts of a
+    row is divided by its own root mean square."""
     out_dtype = out_dtype or a.dtype
-    if not _gpu(a, wa, b, wb):
-        return ref.norm_mix(a, wa, b, wb, eps, ca, cb, out_dtype)
     T, W = a.shape
+    if groups < 1 or W % groups or (groups > 1 and b is not None):
+        raise ValueError(f"norm_mix: {groups} groups must divide the width {W} and go with one input")
+    if not _gpu(a, wa, b, wb):
+        return ref.norm_mix(a, wa, b, wb, eps, ca, cb, out_dtype, groups)
+    if a.stride(1) != 1:
+        raise ValueError("norm_mix: rows must be contiguous")
     if b is not None and (b.shape != a.shape or b.dtype != a.dtype or wb is None):
         raise ValueError("norm_mix: the two inputs must agree in shape and dtype")
     out = torch.empty(T, W, dtype=out_dtype, device=a.device)
-    _native().norm_mix(out.data_ptr(), _p(a), _p(wa, a.dtype, "wa"), _p(b), _p(wb, a.dtype, "wb"), float(eps), float(ca),
-                       float(cb), T, W, _f32(a.dtype), _f32(out_dtype), -1)
+    _native().norm_mix(out.data_ptr(), a.data_ptr(), a.stride(0), _p(wa, a.dtype, "wa"), _p(b), _p(wb, a.dtype, "wb"),
+                       float(eps), float(ca), float(cb), T, W, int(groups), _f32(a.dtype), _f32(out_dtype), -1)
+    return out
+
+
+def postnorm(x: torch.Tensor, branch: Optional[torch.Tensor], alpha: float, gain: float, eps: float, *,
+             branch2: Optional[torch.Tensor] = None, c1: float = 1.0, c2: float = 1.0,
+             out_dtype=None) -> Optional[torch.Tensor]:
+    """Norm after the sum: ``x`` (fp32 [T, W], updated in place) <- rms-norm(alpha x + c1 branch + c2 branch2) * gain
+    with one ``gain`` for the whole row, so the stream itself stays normed.  With ``out_dtype`` the new rows are also
+    returned in that type (the input of the sublayer that reads them next)."""
+    if x.dtype != F32 or not x.is_contiguous():
+        raise TypeError("the residual stream is contiguous fp32")
+    if branch is None and branch2 is not None:
+        branch, branch2, c1, c2 = branch2, None, c2, c1
+    if not _gpu(x, branch, branch2):
+        return ref.postnorm(x, branch, branch2, alpha, c1, c2, gain, eps, out_dtype)
+    T, W = x.shape
+    bt = branch.dtype if branch is not None else out_dtype
+    for t, n in ((branch, "branch"), (branch2, "branch2")):
+        if t is not None and (t.dtype != bt or t.shape != x.shape):
+            raise TypeError(f"postnorm: {n} must be [T, W] of one activation type")
+    if out_dtype is not None and bt is not None and out_dtype != bt:
+        raise TypeError("postnorm: the returned rows take the branches' type")
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    _native().postnorm(_p(x), _p(branch), _p(branch2), float(alpha), float(c1), float(c2), float(gain), float(eps),
+                       _p(out), T, W, _f32(bt or F32), -1)
+    return out
+
+
+def gate_mul(y: torch.Tensor, gate: torch.Tensor, kind: int = GATE_SIGMOID) -> torch.Tensor:
+    """y * sigmoid(gate) (GATE_SIGMOID) or y * silu(gate) (GATE_SILU), element by element; ``y`` [T, F] (the gate's
+    type, or fp32) and ``gate`` [T, F] may be column slices of wider tensors.  Returns [T, F] of the gate's type."""
+    if y.shape != gate.shape or y.dim() != 2:
+        raise ValueError("gate_mul: y and gate must be [T, F]")
+    if not _gpu(y, gate):
+        return ref.gate_mul(y, gate, kind)
+    if y.stride(1) != 1 or gate.stride(1) != 1 or y.dtype not in (gate.dtype, F32):
+        raise ValueError("gate_mul: rows must be contiguous; y is of the gate's type or fp32")
+    T, F = y.shape
+    out = torch.empty(T, F, dtype=gate.dtype, device=y.device)
+    _native().gate_mul(out.data_ptr(), y.data_ptr(), y.stride(0), gate.data_ptr(), gate.stride(0), T, F, int(kind),
+                       int(y.dtype == F32), _f32(gate.dtype), -1)
     return out
 
 
@@ -283,15 +331,22 @@ def wkv_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
 # ----------------------------------------------------------------------------- latent attention
 def latent_kv_write(cache: torch.Tensor, dkv: torch.Tensor, normw: torch.Tensor, q: torch.Tensor,
                     cos_sin: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, C: int, R: int, H: int,
-                    Dn: int, rot_dims: int, eps: float) -> None:
+                    Dn: int, rot_dims: int, eps: float, interleaved: bool = False) -> None:
     """cache[slot] = [rms-norm(dkv[:, :C]) * normw | rotated dkv[:, C:]]; rotates the last R of every head of q
-    ([T, H (Dn + R)]) in place.  ``cos_sin`` [positions, rot_dims] = [cos | sin] fp32."""
+    ([T, H (Dn + R)]) in place.  ``cos_sin`` [positions, rot_dims] = [cos | sin] fp32.  The rotation pairs dimension i
+    with i + rot_dims / 2, or (``interleaved``) dimension 2i with 2i + 1.  ``dkv`` [T, C + R] may be a column slice of
+    a wider projection."""
+    if dkv.dim() != 2 or dkv.shape[1] != C + R:
+        raise ValueError("latent_kv_write: dkv must be [T, C + R]")
     if not _gpu(cache, dkv, q):
-        return ref.latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C, R, H, Dn, rot_dims, eps)
+        return ref.latent_kv_write(cache, dkv, normw, q, cos_sin, positions, slot_mapping, C, R, H, Dn, rot_dims, eps,
+                                   interleaved)
     dt = dkv.dtype
-    _native().latent_kv_write(_p(cache, dt, "cache"), _p(dkv), _p(normw, dt, "normw"), _p(q, dt, "q"),
+    if dkv.stride(1) != 1:
+        raise ValueError("latent_kv_write: rows must be contiguous")
+    _native().latent_kv_write(_p(cache, dt, "cache"), dkv.data_ptr(), _p(normw, dt, "normw"), _p(q, dt, "q"),
                               _p(cos_sin, F32, "cos_sin"), _p(positions, I32), _p(slot_mapping, I32), dkv.shape[0], C,
-                              R, H, Dn, rot_dims, float(eps), _f32(dt), -1)
+                              R, H, Dn, rot_dims, float(eps), _f32(dt), dkv.stride(0), int(bool(interleaved)), -1)
 
 
 LATENT_MFMA = os.environ.get("K8S_LATENT_MFMA", "1") != "0"   # 0: always the plain-FMA attention kernel
@@ -309,15 +364,18 @@ def latent_splits(T: int, H: int, max_keys: int) -> int:
 def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                      tok_seq: torch.Tensor, positions: torch.Tensor, C: int, R: int, H: int, Dn: int, window: int,
                      scale: float, block_size: int, max_keys: int = 0, cu_q: Optional[torch.Tensor] = None,
-                     max_qlen: int = 0) -> torch.Tensor:
+                     max_qlen: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window attention in the latent space over the paged cache; returns softmax-weighted latents [T, H, C].
     ``max_keys``: an upper bound of the keys any token sees (sizes the key splits; 0: the table's capacity).
     ``cu_q`` / ``max_qlen`` (the sequences' query offsets and longest portion): portions of prompts run four
     consecutive tokens per workgroup, sharing the staged cache rows.
+    ``sinks`` [H] fp32: the softmax denominator of head h holds one more term e^sinks[h] (no key, no value).
     bf16 with 16-byte-aligned parts runs on the matrix cores; fp32 and other sizes on the plain-FMA kernel."""
-    if not _gpu(q_abs, q, cache):
+    if sinks is not None and (sinks.dtype != F32 or sinks.numel() != H):
+        raise ValueError("latent_attention: sinks are fp32 [H]")
+    if not _gpu(q_abs, q, cache, sinks):
         return ref.latent_attention(q_abs, q, cache, block_tables, tok_seq, positions, C, R, H, Dn, window, scale,
-                                    block_size, q.dtype)
+                                    block_size, q.dtype, sinks)
     T = q.shape[0]
     dt = q.dtype
     out = torch.empty(T, H, C, dtype=dt, device=q.device)
@@ -336,9 +394,9 @@ def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, 
             pml = torch.empty(T * HP * ns * 2, dtype=F32, device=q.device)
         nseq = cu_q.shape[0] - 1 if cu_q is not None else 0
         nat.latent_attention_mfma(out.data_ptr(), _p(pacc), _p(pml), *args, ns, _p(cu_q, I32, "cu_q"), nseq,
-                                  int(max_qlen), -1)
+                                  int(max_qlen), _p(sinks), -1)
     else:
-        nat.latent_attention(out.data_ptr(), *args, _f32(dt), -1)
+        nat.latent_attention(out.data_ptr(), *args, _f32(dt), _p(sinks), -1)
     return out
 
 
@@ -409,13 +467,16 @@ def window_kv_write(kcache: torch.Tensor, vcache: torch.Tensor, qkv: torch.Tenso
                     D: int, V: int, dims: int, eps: float, unit: bool = True, *,
                     vfirst_in: Optional[torch.Tensor] = None, vfirst_out: Optional[torch.Tensor] = None,
                     lam: float = 0.0, half_layout: bool = False, qnw: Optional[torch.Tensor] = None,
-                    knw: Optional[torch.Tensor] = None) -> None:
+                    knw: Optional[torch.Tensor] = None, head_qnw: Optional[torch.Tensor] = None,
+                    head_knw: Optional[torch.Tensor] = None) -> None:
     """Prepares a projected row [q (H D) | ... k (G D at ``koff``) ... v (G V at ``voff``) ...] of every token: biases,
     rotation of the dimension pairs (2i, 2i + 1), i < dims / 2, by ``cos_sin[pos]`` = [cos | sin] (fp32), unit RMS per
     head of q and k (``unit``), value mixing v <- (1 - lam) v + lam ``vfirst_in`` [T, G V] fp32; the first mixing layer
     leaves its v in ``vfirst_out``.  q is rewritten in place; k and v go to the paged caches [slots, G, D] / [slots, G, V].
     ``half_layout``: the rotation pairs dimension i with i + dims / 2 instead.  ``qnw`` [H D] / ``knw`` [G D]: before the
     rotation the whole projection (all heads at once) is divided by its root mean square and multiplied by the weight.
+    ``head_qnw`` / ``head_knw`` [D]: before the rotation every head is divided by its own root mean square and
+    multiplied by the weight, which all heads share.
     ``kcache`` None (a layer that attends another layer's cache): only the queries are prepared."""
     dt = qkv.dtype
     if kcache is None:
@@ -426,18 +487,23 @@ def window_kv_write(kcache: torch.Tensor, vcache: torch.Tensor, qkv: torch.Tenso
         raise ValueError("window_kv_write: part offsets exceed the projected row")
     if not _gpu(kcache, vcache, qkv):
         return ref.window_kv_write(kcache, vcache, qkv, koff, voff, qb, kb, vb, cos_sin, positions, slot_mapping,
-                                   vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit, half_layout, qnw, knw)
+                                   vfirst_in, vfirst_out, lam, H, G, D, V, dims, eps, unit, half_layout, qnw, knw,
+                                   head_qnw, head_knw)
     T = qkv.shape[0]
     if cos_sin is not None and (cos_sin.shape[1] != dims or cos_sin.dtype != F32):
         raise ValueError("window_kv_write: the angle table must be fp32 [positions, dims]")
     for t in (vfirst_in, vfirst_out):
         if t is not None and (t.shape != (T, G * V) or t.dtype != F32):
             raise ValueError("window_kv_write: mixed values are fp32 [T, G V]")
+    for t in (head_qnw, head_knw):
+        if t is not None and t.numel() != D:
+            raise ValueError("window_kv_write: per-head norm weights are [D]")
     _native().window_kv_write(_p(kcache, dt, "kcache"), _p(vcache, dt, "vcache"), qkv.data_ptr(), qkv.stride(0), koff,
                               voff, _p(qb, dt, "qb"), _p(kb, dt, "kb"), _p(vb, dt, "vb"), _p(cos_sin),
                               _p(positions, I32), _p(slot_mapping, I32), _p(vfirst_in), _p(vfirst_out), float(lam), T, H,
                               G, D, V, dims, float(eps), int(bool(unit)), int(bool(half_layout)), _p(qnw, dt, "qnw"),
-                              _p(knw, dt, "knw"), _f32(dt), -1)
+                              _p(knw, dt, "knw"), _p(head_qnw, dt, "head_qnw"), _p(head_knw, dt, "head_knw"),
+                              _f32(dt), -1)
 
 
 def window_pool(kpool: torch.Tensor, vpool: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
@@ -553,26 +619,45 @@ SCAN_CHUNK_MIN = int(os.environ.get("K8S_SCAN_CHUNK_MIN", "256"))
 def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
                seq_slots: torch.Tensor, positions: torch.Tensor, H: int, D: int, V: int, eps: float, out_dtype, *,
                fbias: Optional[torch.Tensor] = None, ibias: Optional[torch.Tensor] = None,
-               lower: Optional[torch.Tensor] = None, cap: float = 0.0, chunk: Optional[int] = None) -> torch.Tensor:
+               lower: Optional[torch.Tensor] = None, cap: float = 0.0, chunk: Optional[int] = None,
+               aux: Optional[torch.Tensor] = None, head_params: Optional[torch.Tensor] = None,
+               groups: int = 0) -> torch.Tensor:
     """A gated linear recurrence with a matrix state per head over a varlen batch; ``proj`` fp32 [T, ld] is the fused
     input projection with its parts at the column offsets ``cols``; ``state`` [slots, H, record] fp32 is updated in
     place (a portion at position 0 starts from zero).  Returns the normed (and, SCAN_MLSTM, gated) outputs [T, H V].
     SCAN_HGRN2: cols q, f, v; ``lower`` [H D], ``fbias`` [H D], ``normw`` [V].
-    SCAN_MLSTM: cols q, k, v, i, f, g; ``ibias`` / ``fbias`` [H], ``cap`` > 0, ``normw`` [H V]."""
+    SCAN_MLSTM: cols q, k, v, i, f, g; ``ibias`` / ``fbias`` [H], ``cap`` > 0, ``normw`` [H V].
+    SCAN_SSD (a scalar decay per head and token, set by a step size): ``proj`` holds v (the heads' inputs x, H V),
+    k (B) and q (C) (``groups`` D each; head h uses group h // (H / groups)); ``aux`` fp32 [T, lda] holds f (the step
+    size logits, H) and g (the output gate, H V) at ``cols``; ``head_params`` fp32 [3, H] = -exp(A_log), dt_bias, skip.
+    dt = softplus(f + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T; y = (S^T C + skip x) silu(g), returned in fp32
+    without a norm (``normw`` None, ``out_dtype`` fp32)."""
     if proj.dtype != F32 or state.dtype != F32:
         raise TypeError("the recurrence's inputs and state are fp32")
     if proj.dim() != 2 or proj.stride(1) != 1:
         raise ValueError("gated_scan: projected rows must be contiguous")
-    need = {SCAN_HGRN2: ("q", "f", "v"), SCAN_MLSTM: ("q", "k", "v", "i", "f", "g")}[kind]
-    width = {"q": H * D, "k": H * D, "v": H * V, "g": H * V, "i": H, "f": H * D if kind == SCAN_HGRN2 else H}
+    need = {SCAN_HGRN2: ("q", "f", "v"), SCAN_MLSTM: ("q", "k", "v", "i", "f", "g"),
+            SCAN_SSD: ("q", "k", "v", "f", "g")}[kind]
+    G = int(groups) if kind == SCAN_SSD else H
+    width = {"q": G * D, "k": G * D, "v": H * V, "g": H * V, "i": H, "f": H * D if kind == SCAN_HGRN2 else H}
+    if kind == SCAN_SSD:
+        if aux is None or head_params is None or G <= 0 or H % G:
+            raise ValueError("gated_scan: SCAN_SSD needs aux, head_params and groups that divide the heads")
+        if aux.dtype != F32 or aux.stride(1) != 1 or aux.shape[0] != proj.shape[0]:
+            raise TypeError("gated_scan: aux is fp32 [T, lda] with contiguous rows")
+        if head_params.dtype != F32 or head_params.shape != (3, H) or not head_params.is_contiguous():
+            raise TypeError("gated_scan: head_params is contiguous fp32 [3, H]")
+        if out_dtype != F32:
+            raise TypeError("gated_scan: SCAN_SSD returns fp32")
     for key in need:
-        if cols[key] < 0 or cols[key] + width[key] > proj.shape[1]:
+        src = aux if kind == SCAN_SSD and key in ("f", "g") else proj
+        if cols[key] < 0 or cols[key] + width[key] > src.shape[1]:
             raise ValueError(f"gated_scan: part {key!r} exceeds the projected row")
     if state.shape[1:] != (H, gated_scan_record(kind, D, V)):
         raise ValueError("gated_scan: state must be [slots, H, record]")
     if not _gpu(proj, state):
         return ref.gated_scan(proj, kind, cols, fbias, ibias, lower, normw, state, cu_q, seq_slots, positions, H, D, V,
-                              eps, cap, out_dtype)
+                              eps, cap, out_dtype, aux, head_params, G)
     if max(D, V) > gated_scan_max_dim():
         raise ValueError(f"gated_scan: head sizes {D} x {V} exceed the kernel's {gated_scan_max_dim()}")
     T = proj.shape[0]
@@ -585,7 +670,9 @@ def gated_scan(proj: torch.Tensor, kind: int, cols: dict, normw: torch.Tensor, s
     _native().gated_scan(out.data_ptr(), _p(proj), proj.stride(0), kind, c("q"), c("k"), c("v"), c("i"), c("f"), c("g"),
                          _p(fbias, out_dtype, "fbias"), _p(ibias, out_dtype, "ibias"), _p(lower, out_dtype, "lower"),
                          _p(normw, out_dtype, "normw"), _p(state), _p(cu_q, I32), _p(seq_slots, I32),
-                         _p(positions, I32), nseq, H, D, V, float(eps), float(cap), _f32(out_dtype), T, Lc, _p(ws), -1)
+                         _p(positions, I32), nseq, H, D, V, float(eps), float(cap), _f32(out_dtype), T, Lc, _p(ws),
+                         aux.data_ptr() if aux is not None else 0, aux.stride(0) if aux is not None else 0,
+                         _p(head_params), H // G, -1)
     return out
 
 
@@ -596,13 +683,15 @@ CONV_MAX_TAPS = 16
 def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor, tok_seq: torch.Tensor,
                seq_slots: torch.Tensor, positions: torch.Tensor, *, in_bias: Optional[torch.Tensor] = None,
                out_bias: Optional[torch.Tensor] = None, act: int = CONV_NONE, unit_cols: int = 0, unit_dim: int = 0,
-               scale_cols: int = 0, scale: float = 1.0, unit_eps: float = 1e-6) -> torch.Tensor:
+               scale_cols: int = 0, scale: float = 1.0, unit_eps: float = 1e-6, residual: bool = False,
+               out_dtype=F32) -> torch.Tensor:
     """Causal convolution over time per channel over a varlen batch, in fp32.  ``x`` fp32 [T, C] (row stride free),
     ``w`` fp32 [C, taps] (the last tap is the current token's); inputs are x + in_bias, zeros before position 0; the
     taps - 1 inputs before a portion come from ``state`` [slots, taps - 1, C] fp32, which then receives the portion's
     last inputs (a portion at position 0 starts from zeros).  Then out_bias, the activation (CONV_SILU), and, for the
     first ``unit_cols`` channels in groups of ``unit_dim``, v / sqrt(sum(v^2) + unit_eps); the first ``scale_cols``
-    channels times ``scale``.  Returns fp32 [T, C]."""
+    channels times ``scale``.  ``residual``: the token's own input is added to the result (x + conv(x)).  Returns
+    [T, C] in ``out_dtype`` (fp32, or bf16 for a result that feeds a bf16 projection)."""
     T, C = x.shape
     taps = w.shape[1]
     if x.dtype != F32 or w.dtype != F32 or state.dtype != F32 or x.stride(1) != 1:
@@ -615,13 +704,13 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu_q: torc
         raise ValueError("short_conv: scale_cols exceeds the channels")
     if not _gpu(x, w, state):
         return ref.short_conv(x, w, state, cu_q, seq_slots, positions, in_bias, out_bias, act, unit_cols, unit_dim,
-                              scale_cols, scale, unit_eps)
-    out = torch.empty(T, C, dtype=F32, device=x.device)
+                              scale_cols, scale, unit_eps, residual).to(out_dtype)
+    out = torch.empty(T, C, dtype=out_dtype, device=x.device)
     _native().short_conv(out.data_ptr(), x.data_ptr(), x.stride(0), _p(w), _p(state), _p(cu_q, I32, "cu_q"),
                          _p(tok_seq, I32, "tok_seq"), _p(seq_slots, I32, "seq_slots"), _p(positions, I32, "positions"),
                          _p(in_bias, F32, "in_bias"), _p(out_bias, F32, "out_bias"), int(act), T, C, taps,
                          cu_q.shape[0] - 1, int(unit_cols), int(unit_dim), int(scale_cols), float(scale),
-                         float(unit_eps), -1)
+                         float(unit_eps), int(bool(residual)), _f32(out_dtype), -1)
     return out
 
 

@@ -56,6 +56,11 @@ class LatentConfig:
     q_rank: int
     scale: float
     rot_base: float = 10000.0
+    rot_dims: int = -1       # dimensions of the rotated part that turn (the first ones); -1: all of it
+
+    def __post_init__(self):
+        if self.rot_dims < 0:
+            self.rot_dims = self.rot_dim
 
 
 @dataclass
@@ -131,11 +136,9 @@ def _layer_from(l: dict) -> LayerConfig:
     if kind == "latent_attention":
         rot = d.get("rot") or {}
         dim, rot_dim = int(d["dim"]), int(d["rot_dim"])
-        if int(rot.get("dims", rot_dim)) != rot_dim:
-            raise ValueError("latent_attention: the rotated part is rotated whole (rot.dims == rot_dim)")
         mixer: object = LatentConfig(int(d["heads"]), dim, rot_dim, int(d["vdim"]), int(d["kv_rank"]), int(d["q_rank"]),
                                      float(d.get("scale", 1.0 / math.sqrt(dim + rot_dim))),
-                                     float(rot.get("base", 10000.0)))
+                                     float(rot.get("base", 10000.0)), int(rot.get("dims", rot_dim)))
     elif kind == "parallel":
         a, r = d["left"], d["right"]
         dim = int(a["dim"])
@@ -167,7 +170,7 @@ def config_to_json(cfg: SemanexConfig) -> dict:
         m = L.mixer
         if L.type == "latent_attention":
             mixer = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim, "vdim": m.vdim, "kv_rank": m.kv_rank,
-                     "q_rank": m.q_rank, "scale": m.scale, "rot": {"dims": m.rot_dim, "base": m.rot_base}}
+                     "q_rank": m.q_rank, "scale": m.scale, "rot": {"dims": m.rot_dims, "base": m.rot_base}}
         else:
             a, r = m.left, m.right
             mixer = {"left": {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale,
@@ -378,12 +381,12 @@ class SemanexModel(StreamModel):
     def _build_latent(self, get, p: str, m: LatentConfig, where: str) -> _Latent:
         t = self._t
         H, Dn, R, V, C = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
-        if R % 2 or R <= 0:
-            raise ValueError(f"{where}: rot_dim {R} must be even and positive")
+        if m.rot_dims % 2 or not 0 < m.rot_dims <= R:
+            raise ValueError(f"{where}: rot.dims {m.rot_dims} must be even, positive and at most rot_dim {R}")
         w_in, cols = _stack((("dq", get(p + "dq").cpu()), ("dkv", get(p + "dkv").cpu()), ("g", get(p + "g").cpu())))
         return _Latent(m, t(w_in), cols, t(get(p + "dq.norm")), t(get(p + "uq")), t(get(p + "dkv.norm")),
                        t(get(p + "uk").view(H, Dn, C).transpose(1, 2)), t(get(p + "uv").view(H, V, C)),
-                       self._f(get(p + "sink")), t(get(p + "o")), self._rope_table(R, m.rot_base))
+                       self._f(get(p + "sink")), t(get(p + "o")), self._rope_table(m.rot_dims, m.rot_base))
 
     def _build_side(self, get, p: str, m: ParallelConfig, where: str) -> _Side:
         t, f = self._t, self._f
@@ -485,7 +488,7 @@ class SemanexModel(StreamModel):
         cq = sm.norm_mix(proj[:, w.cols["dq"]:w.cols["dq"] + m.q_rank], w.dq_norm, None, None, eps)
         q = sm.linear(cq, w.uq)                                            # [T, H (Dn + R)]
         sm.latent_kv_write(cache, proj[:, w.cols["dkv"]:w.cols["dkv"] + C + R], w.dkv_norm, q, w.cos_sin,
-                           b["positions"], b["slot_mapping"], C, R, H, Dn, R, eps, interleaved=True)
+                           b["positions"], b["slot_mapping"], C, R, H, Dn, m.rot_dims, eps, interleaved=True)
         q_abs = torch.empty(T, H, C, dtype=self.dtype, device=h.device)
         sm.gemm(q.view(T, H, Dn + R)[:, :, :Dn].permute(1, 0, 2), w.uk_t, out=q_abs.permute(1, 0, 2))
         lat = sm.latent_attention(q_abs, q, cache, b["block_tables"], b["tok_seq"], b["positions"], C, R, H, Dn, 0,

@@ -76,7 +76,7 @@ def latent_attention(h, m, w, eps):
     heads; queries come from a normed low-rank row as well."""
     T = h.shape[0]
     H, D, R, V, C = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
-    rot = dict(m["rot"], dims=R)
+    rot = m["rot"]
     cq = rms_unit(h @ w("dq").T, eps) * w("dq.norm")
     q = (cq @ w("uq").T).view(T, H, D + R)
     qn, qr = q[..., :D], rotate_pairs(q[..., D:], rot)
@@ -125,11 +125,10 @@ def ssd(h, m, w, eps):
     decay = torch.exp(-torch.exp(w("A_log")) * dt)                       # [T, H]
     y = torch.zeros(T, H, V, dtype=F64)
     S = torch.zeros(H, N, V, dtype=F64)
+    of = torch.arange(H) // (H // G)                                     # the group of every head
     for t in range(T):
-        for hd in range(H):
-            g = hd // (H // G)
-            S[hd] = decay[t, hd] * S[hd] + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
-            y[t, hd] = S[hd].T @ Cm[t, g] + w("D")[hd] * x[t, hd]
+        S = decay[t, :, None, None] * S + dt[t, :, None, None] * B[t, of][:, :, None] * x[t][:, None, :]
+        y[t] = torch.einsum("hnv,hn->hv", S, Cm[t, of]) + w("D")[:, None] * x[t]
     y = y.reshape(T, inner) * silu(z)
     y = rms_unit(y.view(T, ng, inner // ng), eps).reshape(T, inner) * w("norm")
     return y @ w("o").T
@@ -167,7 +166,20 @@ def forward(tensors, config, tokens, after=None):
         if L.get("mlp"):
             f = gelu_erf(x @ get(p + "mlp.up").T) @ get(p + "mlp.down").T
             x = rms_unit(alpha * x + f, eps) * get(p + "norm2")
+        elif p + "norm2" in tensors:                                       # a second norm without a feed-forward
+            x = rms_unit(alpha * x, eps) * get(p + "norm2")
         if after is not None:
             after.append(x.clone())
     x = rms_unit(x, eps) * get("final.norm")
     return x @ get("head").T
+
+
+def greedy(tensors, config, prompt, n):
+    """n tokens, each the arg-max of the last position's logits (lowest index on a tie)."""
+    toks = list(prompt)
+    out = []
+    for _ in range(n):
+        t = int(torch.argmax(forward(tensors, config, toks)[-1]))
+        out.append(t)
+        toks.append(t)
+    return out

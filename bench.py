@@ -76,9 +76,9 @@ def main() -> int:
                          "decode graphs with the top-p passes")
     ap.add_argument("--model-bench", action="store_true",
                     help="instead of the headline workload: prefill / decode tokens/s of the registered model designs "
-                         "(Putulorn dense, Putulorn with experts, Rupatar, Nukizen, Llama) at equal layer sizes, random weights")
+                         "(Putulorn dense, Putulorn with experts, Rupatar, Nukizen, Semanex, Llama) at equal layer sizes, random weights")
     ap.add_argument("--model-bench-models", default="",
-                    help="(--model-bench) only these rows, comma-separated: putulorn-dense, putulorn-moe, rupatar, nukizen, llama")
+                    help="(--model-bench) only these rows, comma-separated: putulorn-dense, putulorn-moe, rupatar, nukizen, semanex, llama")
     ap.add_argument("--model-bench-widths", default="2048,4096", help="(--model-bench) model widths, comma-separated")
     ap.add_argument("--verbose", action="store_true", help="engine INFO logs (init, autotune, graph capture)")
     args = ap.parse_args()

@@ -27,8 +27,8 @@ struct ScanCols { int q, k, v, i, f, g; };   // column offsets of the parts insi
 // [c CH, (c + 1) CH) of S; group c = 0 prepares each token's per-channel read / keep / write coefficients in LDS (and,
 // KIND 1, owns n).  The partial outputs of the channel groups meet in LDS; group 0 normalises and stores.  The next
 // token's inputs are loaded while the current one is computed; the barriers wait for LDS traffic only.
-// blockDim = (DX, NS): DX = max(D, V) rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest that keeps
-// DX NS within 1024 threads.  State record: S [D][V] (, n [D], m).
+// blockDim = (DX, NS): DX = max(D, V) (KIND 2: V) rounded up to 64, NS = ceil(D / CH), CH (16, 32 or 64) the smallest
+// that keeps DX NS within 1024 threads.  State record: S [D][V] (, n [D], m).
 //
 // MODE 0: a whole portion per workgroup, from the slot's state (zero at position 0) to the slot's state.
 // Long portions run as three passes over chunks of Lc tokens, so the recurrence is parallel over chunks; a chunk record
@@ -81,6 +81,10 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
   }
   const int x = threadIdx.x, c = threadIdx.y, NS = blockDim.y, DX = blockDim.x;
   const bool onv = x < V, ond = x < D;
+  // KIND 2: the block is as wide as the value columns only, and the D shared inputs of a token (B, C) are loaded by the
+  // first ceil(D / DX) thread groups, element c DX + x each
+  const int le = c * DX + x;
+  const bool ldr = KIND == 2 && le < D;
   const int i0 = c * CH;
   const size_t rec = (size_t)D * V + (KIND == 1 ? D + 1 : 0);       // slot record
   const size_t crec = (size_t)D * V + D + 2;                         // chunk record
@@ -131,9 +135,9 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       const float* ar = aux + (size_t)t * ldaux;
       nf = ar[co.f + hd];
       if (MODE != 1 && c == 0 && onv) ng = ar[co.g + (size_t)hd * V + x];
-      if (c == 0 && ond) {
-        if (MODE != 1) nq = r[co.q + qk0 + x];
-        nk = r[co.k + qk0 + x];
+      if (ldr) {
+        if (MODE != 1) nq = r[co.q + qk0 + le];
+        nk = r[co.k + qk0 + le];
       }
       return;
     }
@@ -157,9 +161,9 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
       const float zd = cf + fbh;
       const float dt = fmaxf(zd, 0.f) + log1pf(expf(-fabsf(zd)));
       ka = expf(nega * dt);
-      if (c == 0 && ond) {
-        sq[x] = cq;
-        sb[x] = dt * ck;
+      if (ldr) {
+        sq[le] = cq;
+        sb[le] = dt * ck;
       }
     } else if (KIND == 0) {
       if (c == 0 && ond) {
@@ -342,7 +346,7 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
   if (kind == 2 && (aux == nullptr || hpar == nullptr || R <= 0 || H % R)) return -1;
   if (kind == 0 && lower == nullptr) return -1;
   if (kind == 1 && !(cap > 0.f)) return -1;
-  const int m = D > V ? D : V, DX = (m + 63) / 64 * 64;
+  const int m = (kind == 2 || V > D) ? V : D, DX = (m + 63) / 64 * 64;
   int ch = 16;
   while (ch < 64 && DX * ((D + ch - 1) / ch) > 1024) ch *= 2;
   if (DX * ((D + ch - 1) / ch) > 1024) return -2;

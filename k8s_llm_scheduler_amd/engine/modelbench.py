@@ -1,7 +1,7 @@
 """Prefill and decode throughput of the registered model designs at equal layer sizes (``bench.py --model-bench``).
 
 For every size a Putulorn (dense feed-forwards), a Putulorn with experts, a Rupatar (experts in every layer), a Nukizen
-(dense feed-forward beside every mixer) and a Llama of the same width, depth, feed-forward / expert size and vocabulary are built with random weights and driven through the
+(dense feed-forward beside every mixer), a Semanex (dense feed-forward after every mixer) and a Llama of the same width, depth, feed-forward / expert size and vocabulary are built with random weights and driven through the
 same engine entry points:
 
 * prefill: one whole prompt of ``T`` tokens in one step (``LLMEngine.replay_step``, the varlen forward), tokens/s;
@@ -23,12 +23,21 @@ VOCAB = 32768
 
 
 def _register(width: int) -> Dict[str, str]:
-    from ..models import nukizen, putulorn, rupatar
+    from ..models import nukizen, putulorn, rupatar, semanex
     from ..models.config import PRESETS, LlamaConfig
 
     pairs, ff, wd, heads, eff, experts = SIZES[width]
     names = {"putulorn-dense": f"putulorn-w{width}-dense", "putulorn-moe": f"putulorn-w{width}-moe",
-             "rupatar": f"rupatar-w{width}", "nukizen": f"nukizen-w{width}", "llama": f"llama-w{width}"}
+             "rupatar": f"rupatar-w{width}", "nukizen": f"nukizen-w{width}", "semanex": f"semanex-w{width}",
+             "llama": f"llama-w{width}"}
+    # Semanex: 2 x pairs layers in the order latent, latent, parallel (capped attention + state-space recurrence),
+    # latent; latent attention shaped like Putulorn's (rank 512 + 64 rotated, 128-wide heads) with a query latent of
+    # 3 / 4 of the width, the side attention like Rupatar's (4 query heads per key head, 128-wide), recurrent heads of
+    # 128 state channels x 64 values filling the width, the feed-forward size of the Putulorn-dense layers
+    semanex.PRESETS[names["semanex"]] = semanex.preset(
+        names["semanex"], width, VOCAB, max(1, pairs // 2), heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+        q_rank=width * 3 // 4, side_heads=heads, side_kv_heads=heads // 4, side_dim=128, side_vdim=128,
+        ssd_heads=width // wd, ssd_vdim=wd, ssd_state=128, ssd_groups=max(1, width // wd // 8), norm_groups=4, ff=ff)
     # Nukizen: 2 x pairs layers in the order attention, parallel (attention + delta rule), rglru, attention on the first
     # layer's cache; attention shaped like Rupatar's (4 query heads per key head, 128-wide, chunks of 1024), delta-rule
     # heads of 64 x 64 like the wkv heads, a recurrent unit 5 / 4 of the width in 10 blocks, the dense feed-forward of

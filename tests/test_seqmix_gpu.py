@@ -534,3 +534,157 @@ def test_gated_scan(dt, tol, kind, H, D, V):
                            1e-6, dt, chunk=chunk, **{k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in kw.items()})
         close(o2, oc, tol)
         close(s2, sc, 1e-4)
+
+
+# ----------------------------------------------------------------------------- norms after the sum, gates, grouped norms
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("W", [200, 64, 5000])
+def test_postnorm_and_gates(dt, tol, W):
+    torch.manual_seed(50)
+    x, b1, b2 = torch.randn(T, W) * 2, torch.randn(T, W).to(dt), torch.randn(T, W).to(dt)
+    for kw in (dict(), dict(branch2=b2, c1=1.2, c2=-0.4)):
+        xg, xc = x.to(DEV).clone(), x.clone()
+        og = sm.postnorm(xg, b1.to(DEV), 2.0, 0.8, 1e-6, out_dtype=dt, **{k: _dev(v) for k, v in kw.items()})
+        oc = sm.postnorm(xc, b1, 2.0, 0.8, 1e-6, out_dtype=dt, **kw)
+        close(og, oc, tol)
+        close(xg, xc, 1e-5)
+    xg, xc = x.to(DEV).clone(), x.clone()
+    assert sm.postnorm(xg, None, 1.5, 1.1, 1e-6) is None and sm.postnorm(xc, None, 1.5, 1.1, 1e-6) is None
+    close(xg, xc, 1e-5)
+    close(sm.postnorm(xg, None, 1.0, 0.5, 1e-6, out_dtype=dt), sm.postnorm(xc, None, 1.0, 0.5, 1e-6, out_dtype=dt), tol)
+    # gates on column slices of wider tensors; an fp32 input gated into the activation type
+    F = min(W, 300)
+    wide, y = (torch.randn(T, F + 24) * 2).to(dt), torch.randn(T, F + 8)
+    for kind in (sm.GATE_SIGMOID, sm.GATE_SILU):
+        for yy in (y[:, 8:], y[:, :F].to(dt)):
+            close(sm.gate_mul(yy.to(DEV), wide.to(DEV)[:, 16:16 + F], kind), sm.gate_mul(yy, wide[:, 16:16 + F], kind), tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("W,groups", [(192, 1), (192, 4), (70, 7), (96, 96), (640, 2)])
+def test_norm_of_a_slice_in_groups(dt, tol, W, groups):
+    torch.manual_seed(51)
+    wide = torch.randn(T, W + 40)
+    w = 1 + 0.2 * torch.randn(W)
+    for a, ww in ((wide[:, 24:24 + W], w), (wide.to(dt)[:, 24:24 + W], w.to(dt))):
+        og = sm.norm_mix(a.to(DEV), ww.to(DEV), None, None, 1e-5, ca=0.7, out_dtype=dt, groups=groups)
+        close(og, sm.norm_mix(a, ww, None, None, 1e-5, ca=0.7, out_dtype=dt, groups=groups), tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("taps,C", [(3, 70), (1, 64), (8, 300)])
+def test_short_conv_with_residual(dt, tol, taps, C):
+    """x + conv(x) in the activation type, twice, so that the second call reads the inputs the first one saved."""
+    torch.manual_seed(52)
+    cu, pos, slots, tok_seq = batch()
+    w = torch.randn(C, taps)
+    state = torch.randn(4, max(taps - 1, 0), C)
+    sc, sg = state.clone(), state.to(DEV).clone()
+    x = torch.randn(T, C)
+    for step in range(2):
+        oc = sm.short_conv(x, w, sc, cu, tok_seq, slots, pos, residual=True, out_dtype=dt)
+        og = sm.short_conv(x.to(DEV), w.to(DEV), sg, cu.to(DEV), tok_seq.to(DEV), slots.to(DEV), pos.to(DEV),
+                           residual=True, out_dtype=dt)
+        assert og.dtype == dt
+        close(og, oc, tol)
+        close(sg, sc, 1e-6)
+        cu = torch.tensor([0, 2, 3, 3, 4], dtype=torch.int32)
+        pos = torch.tensor([9, 10, 6, 30], dtype=torch.int32)
+        tok_seq = torch.tensor([0, 0, 1, 3], dtype=torch.int32)
+        x = torch.randn(4, C)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,Dn,R,C,dims", [(6, 40, 24, 72, 24), (3, 16, 8, 130, 4), (20, 16, 8, 48, 8), (16, 32, 16, 64, 16),
+                                           (1, 2, 2, 1, 2)])
+def test_latent_attention_interleaved_pairs_and_sinks(dt, tol, H, Dn, R, C, dims):
+    """The latent row as a slice of a wider projection, the rotation of the pairs (2i, 2i + 1), and a learned term per
+    head in the softmax's denominator: per token, four tokens per workgroup, and few tokens with key splits."""
+    torch.manual_seed(53)
+    cu, pos, slots, tok_seq = batch()
+    bs, per = 16, 2
+    L = C + R
+    cache = torch.randn(4 * per * bs, L).to(dt)
+    bt = torch.randperm(4 * per).view(4, per).int()
+    slot_map = torch.tensor([int(bt[tok_seq[t], pos[t] // bs]) * bs + int(pos[t]) % bs for t in range(T)],
+                            dtype=torch.int32)
+    wide, nw = torch.randn(T, L + 48).to(dt), (1 + 0.1 * torch.randn(C)).to(dt)
+    q = torch.randn(T, H * (Dn + R)).to(dt)
+    cs = ref.rope_table(dims, 64, 10000.0)
+    cg, qg, cc, qc = cache.to(DEV).clone(), q.to(DEV).clone(), cache.clone(), q.clone()
+    sm.latent_kv_write(cg, wide.to(DEV)[:, 32:32 + L], nw.to(DEV), qg, cs.to(DEV), pos.to(DEV), slot_map.to(DEV), C, R, H,
+                       Dn, dims, 1e-6, interleaved=True)
+    sm.latent_kv_write(cc, wide[:, 32:32 + L], nw, qc, cs, pos, slot_map, C, R, H, Dn, dims, 1e-6, interleaved=True)
+    close(cg, cc, tol)
+    close(qg, qc, tol)
+    half = q.clone()
+    sm.latent_kv_write(cache.clone(), wide[:, 32:32 + L], nw, half, cs, pos, slot_map, C, R, H, Dn, dims, 1e-6)
+    assert dims == 2 or not torch.allclose(half.float(), qc.float(), atol=1e-2)   # the pair layout matters
+    qabs = torch.randn(T, H, C).to(dt) * 0.3
+    sinks = torch.randn(H) * 2
+    sinks[0] = 9.0                                                            # above every score
+    oc = sm.latent_attention(qabs, qc, cc, bt, tok_seq, pos, C, R, H, Dn, 0, 0.2, bs, sinks=sinks)
+    assert not torch.allclose(oc.float(), sm.latent_attention(qabs, qc, cc, bt, tok_seq, pos, C, R, H, Dn, 0, 0.2, bs).float(),
+                              atol=1e-2)
+    for kw in ({}, {"cu_q": cu.to(DEV), "max_qlen": 27}):
+        og = sm.latent_attention(qabs.to(DEV), qc.to(DEV), cc.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H,
+                                 Dn, 0, 0.2, bs, sinks=sinks.to(DEV), **kw)
+        close(og, oc, tol)
+    few = torch.tensor([3, 20, 30], dtype=torch.long)                         # few tokens: key splits and their merge
+    og = sm.latent_attention(qabs[few].to(DEV), qc[few].to(DEV), cc.to(DEV), bt.to(DEV), tok_seq[few].to(DEV),
+                             pos[few].to(DEV), C, R, H, Dn, 0, 0.2, bs, 64, sinks=sinks.to(DEV))
+    close(og, oc[few], tol)
+
+
+@pytest.mark.parametrize("dt,tol", DTYPES)
+@pytest.mark.parametrize("H,G,D,V", [(8, 4, 32, 128), (3, 1, 20, 12), (6, 3, 80, 72), (16, 4, 128, 64)])
+def test_per_head_normed_queries_and_keys(dt, tol, H, G, D, V):
+    torch.manual_seed(54)
+    cu, pos, slots, tok_seq = batch()
+    bs = 16
+    n = 8 * bs
+    koff, voff = H * D + 16, H * D + 16 + G * D
+    proj = torch.randn(T, voff + G * V + 5).to(dt)
+    slot_map = torch.randperm(n)[:T].int()
+    qw, kw_ = (1 + 0.3 * torch.randn(D)).to(dt), (1 + 0.3 * torch.randn(D)).to(dt)
+    out = {}
+    for dev in ("cpu", DEV):
+        kc, vc = torch.zeros(n, G, D, dtype=dt, device=dev), torch.zeros(n, G, V, dtype=dt, device=dev)
+        p = proj.to(dev).clone()
+        sm.window_kv_write(kc, vc, p, koff, voff, None, None, None, None, pos.to(dev), slot_map.to(dev), H, G, D, V, 0,
+                           1e-6, False, head_qnw=qw.to(dev), head_knw=kw_.to(dev))
+        out[dev] = (kc, vc, p)
+    for a, b in zip(out[DEV], out["cpu"]):
+        close(a, b, tol)
+    q = out["cpu"][2][:, :H * D].float().view(T, H, D)
+    ratio = q.pow(2).mean(-1).sqrt() / (qw.float().pow(2).mean().sqrt())
+    assert (ratio - 1).abs().max() < 0.35                                     # every head normed by itself
+
+
+# ----------------------------------------------------------------------------- state-space recurrence
+@pytest.mark.parametrize("H,G,N,V", [(4, 2, 16, 24), (8, 4, 40, 56), (3, 1, 100, 5), (2, 2, 128, 64), (6, 3, 64, 128),
+                                     (1, 1, 256, 200), (5, 5, 7, 70)])
+def test_ssd_scan(H, G, N, V):
+    torch.manual_seed(55)
+    cu, pos, slots, _ = batch()
+    inner = H * V
+    cols = {"v": 2, "k": 2 + inner + 1, "q": 2 + inner + 1 + G * N + 3, "g": 1, "f": 1 + inner + 5}
+    xbc = torch.randn(T, cols["q"] + G * N + 2)
+    aux = torch.randn(T, cols["f"] + H + 3) * 1.5
+    hp = torch.stack([-torch.exp(torch.randn(H) * 0.7 - 1.0), torch.randn(H), torch.randn(H)]).contiguous()
+    state = torch.randn(4, H, N * V) * 0.5
+    sc, sg = state.clone(), state.to(DEV).clone()
+    args = lambda d, s: (xbc.to(d), sm.SCAN_SSD, cols, None, s, cu.to(d), slots.to(d), pos.to(d), H, N, V, 1e-6,
+                         torch.float32)
+    kw = lambda d: dict(aux=aux.to(d), head_params=hp.to(d), groups=G)
+    oc = sm.gated_scan(*args("cpu", sc), **kw("cpu"))
+    og = sm.gated_scan(*args(DEV, sg), **kw(DEV))
+    assert og.dtype == torch.float32
+    close(og, oc, 2e-5)
+    close(sg, sc, 1e-4)
+    assert torch.equal(sg[1].cpu(), state[1])                                  # the empty sequence's slot
+    for chunk in (4, 7, 16, 64):                       # three passes over chunks: same outputs, same final states
+        s2 = state.to(DEV).clone()
+        o2 = sm.gated_scan(*args(DEV, s2), chunk=chunk, **kw(DEV))
+        close(o2, oc, 2e-5)
+        close(s2, sc, 1e-4)

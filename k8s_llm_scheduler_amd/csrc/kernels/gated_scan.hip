@@ -271,7 +271,7 @@ __global__ __launch_bounds__(1024) void gated_scan_kernel(TA* __restrict__ out, 
 
 // Start states of a sequence's chunks from the slot's state (zero at position 0: chunk 0 has no record then) and the
 // chunks' records.
-// One workgroup per (sequence, head); every thread walks the chunks for its elements of (S, n).
+// Workgroups (sequence, head, slice of the record's elements); every thread walks the chunks for its elements of (S, n).
 template <int KIND>
 __global__ void gated_prefix_kernel(float* __restrict__ cs_start, const float* __restrict__ cs_loc,
                                     const float* __restrict__ state, const int* __restrict__ cu_q,
@@ -293,7 +293,7 @@ __global__ void gated_prefix_kernel(float* __restrict__ cs_start, const float* _
   const float* st = state + ((size_t)seq_slots[s] * H + hd) * rec;
   const int nel = KIND == 1 ? DV + D : DV;
   float* own = cs_start + ((size_t)first * H + hd) * crec;        // chunk 0 starts from a copy of the slot's record
-  for (int e = threadIdx.x; e < nel; e += blockDim.x) {
+  for (int e = blockIdx.z * blockDim.x + threadIdx.x; e < nel; e += blockDim.x * gridDim.z) {
     float X = zero ? 0.f : st[e];
     float m = (KIND == 1 && !zero) ? st[DV + D] : 0.f;
     if (!zero) {
@@ -381,10 +381,14 @@ extern "C" int k8s_gated_scan(void* out, const float* proj, long ld, int kind, i
   float* loc = ws;
   float* start = ws + (size_t)chunks * H * ((size_t)D * V + D + 2);
   K8S_GS_T(1, chunks, loc, nullptr);
+  // a record's elements walk the chunks independently of each other: at most four per thread
+  int pz = (D * V + D + 1023) / 1024;
+  pz = pz < 1 ? 1 : (pz > 64 ? 64 : pz);
+  const dim3 pgrid(nseq, H, pz);
   if (kind != 1)     // one decay per key channel (KIND 2: the head's, repeated)
-    gated_prefix_kernel<0><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+    gated_prefix_kernel<0><<<pgrid, 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
   else
-    gated_prefix_kernel<1><<<dim3(nseq, H), 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
+    gated_prefix_kernel<1><<<pgrid, 256, 0, s>>>(start, loc, state, cu_q, seq_slots, positions, H, D, V, Lc);
   K8S_GS_T(2, chunks, nullptr, start);
 #undef K8S_GS_T
 #undef K8S_GS_K

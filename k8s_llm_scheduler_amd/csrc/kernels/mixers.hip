@@ -433,19 +433,52 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
   for (int n = 0; n < NDB; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
   const int qd = li >> 2, pd = li & 3;
+  // NWV = 4: the cache rows of the next step are loaded into registers under the MFMAs of the current one (PF 16-byte
+  // pieces per thread cover 32 rows of up to 32 NKK elements); the LDS tile is written from them at the next step's start.
+  constexpr int PF = NWV == 4 ? NKK / 2 : 0;
+  u32x4 pf[PF > 0 ? PF : 1];
+  auto fetch = [&](int tile) {
+    const int j0 = lo_min + tile * 32;
+#pragma unroll
+    for (int k = 0; k < PF; ++k) {
+      const int idx = tid + k * 64 * NWV;
+      u32x4 v = zero;
+      if (idx < 32 * cpr) {
+        const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
+        if (key <= p_last) {
+          const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
+          v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
+        }
+      }
+      pf[k] = v;
+    }
+  };
+  if (PF > 0 && t0 < t1) fetch(t0);
   for (int tile = t0; tile < t1; ++tile) {
     const int j0 = lo_min + tile * 32;
     __syncthreads();
-    for (int idx = tid; idx < 32 * cpr; idx += 64 * NWV) {
-      const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
-      u32x4 v = zero;
-      if (key <= p_last) {
-        const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
-        v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
+    if (PF > 0) {
+#pragma unroll
+      for (int k = 0; k < PF; ++k) {
+        const int idx = tid + k * 64 * NWV;
+        if (idx < 32 * cpr) {
+          const int r = idx / cpr, c = idx - r * cpr;
+          *reinterpret_cast<u32x4*>(klds + r * rowb + 16 * c) = pf[k];
+        }
       }
-      *reinterpret_cast<u32x4*>(klds + r * rowb + 16 * c) = v;
+    } else {
+      for (int idx = tid; idx < 32 * cpr; idx += 64 * NWV) {
+        const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
+        u32x4 v = zero;
+        if (key <= p_last) {
+          const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
+          v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
+        }
+        *reinterpret_cast<u32x4*>(klds + r * rowb + 16 * c) = v;
+      }
     }
     __syncthreads();
+    if (PF > 0 && tile + 1 < t1) fetch(tile + 1);
     if (!valid || j0 > p || j0 + 31 < lo) continue;     // no key of this step is visible to this wave's token
     f32x4 sacc[2];
 #pragma unroll

@@ -14,9 +14,9 @@ lists.  What a mixer reads first passes a short causal convolution over time per
 * ``parallel``: two mixers side by side on the same input, ``left_scale * left + right_scale * right``.  Left:
   grouped-query attention without positions; queries and keys RMS-normed per head with a weight of ``dim`` numbers that
   the heads share; scores ``q . k * scale`` capped to ``cap tanh(s / cap)``; causal softmax; output times
-  ``sigmoid(W_g h)`` before ``W_o``.  Right: a state-space recurrence with a scalar decay per head
-  (Mamba-2: "Transformers are SSMs", Dao and Gu): ``W_in h = [z | x | B | C | dt]``; x, B, C pass a short causal convolution with bias and silu;
-  ``dt = softplus(dt + dt_bias)``; per head (B, C of its group) ``S <- exp(-exp(A_log) dt) S + dt B x^T``,
+  ``sigmoid(W_g h)`` before ``W_o``.  Right: a state-space recurrence with a scalar decay per head (the Mamba-2 layer
+  of "Transformers are SSMs", Dao and Gu): ``W_in h = [z | x | B | C | dt]``; x, B, C pass a short causal convolution
+  with bias and silu; ``dt = softplus(dt + dt_bias)``; per head (B, C of its group) ``S <- exp(-exp(A_log) dt) S + dt B x^T``,
   ``y = S^T C + D x``; ``y silu(z)`` is RMS-normed in ``norm_groups`` equal parts, times a weight, then ``W_o``.
 
 The model presents the engine's interface through :class:`~.stream.StreamModel`; caches: per latent attention a paged
@@ -247,7 +247,7 @@ def preset(name: str, width: int, vocab: int, repeats: int, *, heads: int, dim: 
            q_rank: int, side_heads: int, side_kv_heads: int, side_dim: int, side_vdim: int, ssd_heads: int,
            ssd_vdim: int, ssd_state: int, ssd_groups: int, norm_groups: int, ff: int, taps: int = 4,
            order=("latent_attention", "latent_attention", "parallel", "latent_attention")) -> SemanexConfig:
-    """``repeats`` x ``order``, every layer with a feed-forward."""
+    """``repeats`` x ``order``, every layer with a feed-forward; alpha grows with the depth as (2 layers)^(1/4)."""
     layers: List[LayerConfig] = []
     for _ in range(repeats):
         for kind in order:
@@ -259,8 +259,8 @@ def preset(name: str, width: int, vocab: int, repeats: int, *, heads: int, dim: 
                                                     1.0 / math.sqrt(side_dim), 30.0),
                                        SsdConfig(ssd_heads, ssd_vdim, ssd_state, ssd_groups, norm_groups, 4), 1.0, 1.0)
             layers.append(LayerConfig(kind, mixer, ff))
-    return SemanexConfig(name, vocab, width, layers, rms_eps=1e-6, alpha=(2.0 * len(layers)) ** 0.25, embed_scale=math.sqrt(width),
-                         canon_taps=taps)
+    return SemanexConfig(name, vocab, width, layers, rms_eps=1e-6, alpha=(2.0 * len(layers)) ** 0.25,
+                         embed_scale=math.sqrt(width), canon_taps=taps)
 
 
 PRESETS = {

@@ -3,8 +3,6 @@ and generation entry points) against the plain float64 oracle in semanex_oracle.
 (reference ops: model, cache, state and scheduler logic) and, marked gpu, on the HIP kernels.  Small own
 configurations, random weights; where random weights would hide a fault the weights are shaped so that it shows."""
 
-import copy
-
 import pytest
 import torch
 

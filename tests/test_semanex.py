@@ -621,3 +621,64 @@ def test_random_configurations(tmp_path, device, seed):
         ga.append(rows[:1])
     assert rel_err(torch.cat(ga), wa) < TOL["float32"], cfg
     assert rel_err(torch.cat(gb), wb) < TOL["float32"], cfg
+
+
+def mid_config(seed):
+    """A random model of a few hundred channels: up to 24 heads, latent ranks up to 160, recurrent states up to 128
+    channels, feed-forwards of one to two widths -- the sizes at which the matrix-core kernels and the tuned products
+    take over."""
+    import random
+
+    rng = random.Random(seed)
+    pick = lambda xs: rng.choice(xs)
+    width = pick([128, 192, 256, 320, 384])
+    layers = []
+    for _ in range(rng.randint(2, 4)):
+        ff = pick([0, width, 2 * width, 3 * width // 2])
+        if rng.random() < 0.55:
+            layers.append(latent(ff=ff, heads=pick([2, 4, 6, 12, 16, 24]), dim=pick([16, 32, 48, 96]),
+                                 rot_dim=pick([8, 16, 64]), vdim=pick([16, 32, 64, 128]),
+                                 kv_rank=pick([32, 48, 96, 128, 160]), q_rank=pick([48, 64, 192]),
+                                 scale=pick([0.08, 0.1, 0.15]), base=pick([1e4, 1e6, 5e5])))
+        else:
+            kv, g = pick([1, 2, 4]), pick([1, 2, 4])
+            heads = g * pick([1, 2, 4])
+            layers.append(parallel(ff=ff, left=capped(heads=kv * pick([1, 2, 4]), kv_heads=kv, dim=pick([32, 64, 128]),
+                                                      vdim=pick([32, 64, 128]), scale=pick([0.09, 0.125]),
+                                                      softcap=pick([10.0, 50.0])),
+                                   right=ssd(heads=heads, vdim=pick([16, 32, 48, 64]), state=pick([16, 32, 64, 128]),
+                                             groups=g, norm_groups=pick([1, 2, heads]), conv=pick([2, 3, 4])),
+                                   left_scale=pick([0.8, 1.2]), right_scale=pick([0.7, 1.0])))
+    return config(layers, width=width, vocab=pick([300, 512, 1000]), eps=1e-6, alpha=pick([1.7, 2.0, 2.5]),
+                  taps=pick([2, 3, 5]), scale=width ** 0.5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(6))
+def test_mid_size_configurations_on_the_kernels(tmp_path, dtype, seed):
+    """A 290-token prompt (long enough for the chunk-parallel recurrence), a short portion, a second request beside
+    decoded tokens.  bfloat16: nine rows in ten within the tolerance (single rows of random networks amplify rounding)."""
+    cfg = mid_config(seed)
+    eng, tensors = make(tmp_path, cfg, "cuda", dtype, seed=seed, max_tokens=448, slots=4)
+    V = cfg["vocab"]
+    a, b = tokens(320, V, 100 + seed), tokens(50, V, 200 + seed)
+    wa, wb = expect(cfg, tensors, a), expect(cfg, tensors, b)
+    ga = [eng.replay_step([("a", a[:290], list(range(290)))]), eng.replay_step([("a", a[290:293], [0, 1, 2])])]
+    gb = []
+    for i in range(293, 320):
+        if i == 300:
+            rows = eng.replay_step([("a", [a[i]], [0]), ("b", b[:40], list(range(40)))])
+            gb.append(rows[1:])
+        elif 300 < i <= 310:
+            rows = eng.replay_step([("a", [a[i]], [0]), ("b", [b[40 + i - 301]], [0])], ["b"] if i == 310 else [])
+            gb.append(rows[1:])
+        else:
+            rows = eng.replay_step([("a", [a[i]], [0])])
+        ga.append(rows[:1])
+    for got, want in ((torch.cat(ga), wa), (torch.cat(gb), wb)):
+        e = row_errs(got, want)
+        if dtype == "float32":
+            assert e.max().item() < TOL[dtype], cfg
+        else:
+            assert int((e >= TOL[dtype]).sum()) <= e.numel() // 10 and e.median().item() < 2e-2, cfg

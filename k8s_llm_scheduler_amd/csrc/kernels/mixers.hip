@@ -365,17 +365,19 @@ typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 // NWV = 4: one workgroup per (4 consecutive tokens of a sequence, head group); the waves share every staged key step
 // (the union of their windows) and mask their own range, so a prompt reads each cached row once per 4 queries.
 // The queries stay in registers (NKK 32-wide pieces of [q_abs | q_rot] per lane).
-template <int NDB, int NKK, int NWV>
+// EX: the sizes fill the template's bounds exactly (C == 16 NDB, C + R == 32 NKK), so the unrolled loops hold no
+// branches and the LDS reads of a step are issued ahead of the MFMAs that consume them.
+template <int NDB, int NKK, int NWV, bool EX>
 __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ pacc, float* __restrict__ pml, const bf16_t* __restrict__ q_abs,
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ cu_q, int C, int R,
-    int H, int Dn, int window, float scale, int bs, int nsplit, const float* __restrict__ sinks) {
+    int H, int Dn, int window, float scale, int bs, int nsplit, const float* __restrict__ sinks, int bt_lds) {
   extern __shared__ __attribute__((aligned(16))) char smem_b[];
-  char* klds = smem_b;               // [32][L + 8] bf16
+  char* klds = smem_b;               // [32][L + 8] bf16; then (bt_lds) the block-table entries of the keys this block reads
   const int hg = blockIdx.y;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 15, g = lane >> 4;
-  const int L = C + R, rowb = (L + 8) * 2, ndb = C / 16, HP = gridDim.y * 16;
+  const int L = C + R, rowb = (L + 8) * 2, ndb = EX ? NDB : C / 16, HP = gridDim.y * 16;
   int t, split, seq, p_first, p_last;
   bool valid;
   if (NWV == 1) {
@@ -410,9 +412,17 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
   const int tps = (ntiles + nsplit - 1) / nsplit;
   const int t0 = split * tps, t1 = min(ntiles, t0 + tps);
   const int* btr = block_tables + (size_t)seq * max_blocks;
-  const int cpr = L / 8;             // 16-byte chunks per row
+  const int cpr = EX ? 4 * NKK : L / 8;   // 16-byte chunks per row
   const u32x4 zero = u32x4{0u, 0u, 0u, 0u};
-  const int nkk = (L + 31) / 32;
+  const int nkk = EX ? NKK : (L + 31) / 32;
+  // NWV = 4: the block-table entries go to LDS once, so a step's row addresses do not wait for a global load each
+  int* bts = reinterpret_cast<int*>(smem_b + 32 * rowb);
+  const int b0 = lo_min / bs;
+  const bool bt_staged = NWV == 4 && bt_lds != 0;
+  if (bt_staged) {
+    for (int i = tid; i <= p_last / bs - b0; i += 64 * NWV) bts[i] = btr[b0 + i];
+    __syncthreads();
+  }
   // B operand of S^T = K Q^T: lane (li = head, g) holds q[head][32 kk + 8 g .. + 7]
   bf16x8 qf[NKK];
   {
@@ -435,7 +445,7 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
   const int qd = li >> 2, pd = li & 3;
   // NWV = 4: the cache rows of the next step are loaded into registers under the MFMAs of the current one (PF 16-byte
   // pieces per thread cover 32 rows of up to 32 NKK elements); the LDS tile is written from them at the next step's start.
-  constexpr int PF = NWV == 4 ? NKK / 2 : 0;
+  constexpr int PF = NWV == 4 ? (NKK + 1) / 2 : 0;
   u32x4 pf[PF > 0 ? PF : 1];
   auto fetch = [&](int tile) {
     const int j0 = lo_min + tile * 32;
@@ -446,7 +456,8 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
       if (idx < 32 * cpr) {
         const int r = idx / cpr, c = idx - r * cpr, key = j0 + r;
         if (key <= p_last) {
-          const size_t slot = (size_t)btr[key / bs] * bs + (key % bs);
+          const int kb = key / bs;
+          const size_t slot = (size_t)(bt_staged ? bts[kb - b0] : btr[kb]) * bs + (key - kb * bs);
           v = *reinterpret_cast<const u32x4*>(cache + slot * L + 8 * c);
         }
       }
@@ -489,7 +500,7 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
         if (kk < nkk) {
           const int piece = 32 * kk + 8 * g;
           bf16x8 ka = __builtin_bit_cast(bf16x8, zero);
-          if (piece < L) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowb + 2 * piece);
+          if (EX || piece < L) ka = *reinterpret_cast<const bf16x8*>(klds + (16 * m + li) * rowb + 2 * piece);
           acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[kk], acc, 0, 0, 0);
         }
       }
@@ -508,13 +519,13 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
     const float m_new = fmaxf(m_run, tmax);       // finite: the step holds a visible key
-    const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+    const float alpha = m_run == -INFINITY ? 0.f : __expf(m_run - m_new);
     float rsum = 0.f;
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = expf(sacc[m][i] - m_new);
+        const float pv = __expf(sacc[m][i] - m_new);     // the weights are rounded to bf16 for the product
         sacc[m][i] = pv;
         rsum += pv;
       }
@@ -522,9 +533,16 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
     rsum += __shfl_xor(rsum, 32, WAVE);
     l_run = l_run * alpha + rsum;
     m_run = m_new;
-    float a_i[4];
+    // the running maxima settle after the first steps: the accumulators are rescaled only when some head's moved
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+      float a_i[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g * 4 + i, WAVE);
+      for (int i = 0; i < 4; ++i) a_i[i] = __shfl(alpha, g * 4 + i, WAVE);
+#pragma unroll
+      for (int n = 0; n < NDB; ++n)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[n][i] *= a_i[i];
+    }
     bf16x8 pa;       // slot j < 4: key 4 g + j; slot j >= 4: key 16 + 4 g + (j - 4)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -535,8 +553,6 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
 #pragma unroll
     for (int n = 0; n < NDB; ++n) {
       if (n < ndb) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[n][i] *= a_i[i];
         const int col = 16 * n + 4 * pd;
         const bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(klds + r0 * rowb + 2 * col));
         const bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(klds + r1 * rowb + 2 * col));
@@ -740,24 +756,31 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
   if (!k8s_latent_mfma_ok(C, R, Dn) || H <= 0 || bs <= 0 || nsplit < 1 || (nsplit > 1 && (!pacc || !pml))) return -1;
   const int L = C + R, HG = (H + 15) / 16;
   const size_t lds = (size_t)32 * (L + 8) * 2;
+  const int bt_lds = (size_t)max_blocks * sizeof(int) <= 24576;     // the block table of one sequence beside the key tile
+  const size_t bt_bytes = bt_lds ? (size_t)max_blocks * sizeof(int) : 0;
   const bool tiles = nsplit == 1 && cu_q != nullptr && nseq > 0 && max_qlen > 1;
   if (tiles && nseq > 65535) return -2;
   const dim3 grid = tiles ? dim3((max_qlen + 3) / 4, HG, nseq) : dim3(T, HG, nsplit);
-#define K8S_LM(NDB, NKK)                                                                                              \
+#define K8S_LM(NDB, NKK, EX)                                                                                            \
   do {                                                                                                                \
     if (tiles)                                                                                                        \
-      latent_attention_mfma_kernel<NDB, NKK, 4><<<grid, 256, lds, s>>>(                                               \
+      latent_attention_mfma_kernel<NDB, NKK, 4, EX><<<grid, 256, lds + bt_bytes, s>>>(                                             \
           (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
-          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks);                       \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks, bt_lds);               \
     else                                                                                                              \
-      latent_attention_mfma_kernel<NDB, NKK, 1><<<grid, 64, lds, s>>>(                                                \
+      latent_attention_mfma_kernel<NDB, NKK, 1, EX><<<grid, 64, lds, s>>>(                                             \
           (bf16_t*)out, pacc, pml, (const bf16_t*)q_abs, (const bf16_t*)q, (const bf16_t*)cache, block_tables,        \
-          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks);                       \
+          max_blocks, tok_seq, positions, cu_q, C, R, H, Dn, window, scale, bs, nsplit, sinks, 0);                    \
   } while (0)
-  if (C <= 128 && L <= 256) K8S_LM(8, 8);
-  else if (C <= 256 && L <= 256) K8S_LM(16, 8);
-  else if (C <= 256) K8S_LM(16, 20);
-  else K8S_LM(32, 20);
+  if (C == 512 && L == 576) K8S_LM(32, 18, true);        // sizes that fill an instantiation exactly
+  else if (C == 256 && L == 320) K8S_LM(16, 10, true);
+  else if (C == 128 && L == 192) K8S_LM(8, 6, true);
+  else if (C == 128 && L == 160) K8S_LM(8, 5, true);
+  else if (C == 64 && L == 96) K8S_LM(4, 3, true);
+  else if (C <= 128 && L <= 256) K8S_LM(8, 8, false);
+  else if (C <= 256 && L <= 256) K8S_LM(16, 8, false);
+  else if (C <= 256) K8S_LM(16, 20, false);
+  else K8S_LM(32, 20, false);
 #undef K8S_LM
   if (nsplit > 1)
     latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit,

@@ -596,7 +596,8 @@ def test_short_conv_with_residual(dt, tol, taps, C):
 
 @pytest.mark.parametrize("dt,tol", DTYPES)
 @pytest.mark.parametrize("H,Dn,R,C,dims", [(6, 40, 24, 72, 24), (3, 16, 8, 130, 4), (20, 16, 8, 48, 8), (16, 32, 16, 64, 16),
-                                           (1, 2, 2, 1, 2)])
+                                           (1, 2, 2, 1, 2), (4, 16, 64, 256, 64), (18, 16, 64, 128, 32), (4, 24, 32, 128, 32),
+                                           (5, 16, 32, 64, 32), (16, 64, 64, 512, 64)])
 def test_latent_attention_interleaved_pairs_and_sinks(dt, tol, H, Dn, R, C, dims):
     """The latent row as a slice of a wider projection, the rotation of the pairs (2i, 2i + 1), and a learned term per
     head in the softmax's denominator: per token, four tokens per workgroup, and few tokens with key splits."""

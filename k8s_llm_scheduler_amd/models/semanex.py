@@ -395,12 +395,15 @@ class SemanexModel(StreamModel):
             raise ValueError(f"{where}: {a.heads} query heads over {a.kv_heads} key / value heads")
         if r.heads % r.groups or r.inner % r.norm_groups:
             raise ValueError(f"{where}: {r.groups} groups / {r.norm_groups} norm groups do not divide the {r.heads} heads")
-        if max(r.state, r.vdim) > sm.gated_scan_max_dim() or r.conv > sm.CONV_MAX_TAPS:
-            raise ValueError(f"{where}: state {r.state} x {r.vdim} or {r.conv} taps exceed the kernels'")
+        if max(r.state, r.vdim) > sm.gated_scan_max_dim():
+            raise ValueError(f"{where}: state {r.state} x {r.vdim} exceeds the kernels' {sm.gated_scan_max_dim()}")
         q = p + "left."
         w_in, cols = _stack(tuple((s, get(q + s).cpu()) for s in ("q", "k", "v", "g")))
         left = _Capped(a, t(w_in), cols, t(get(q + "q.norm")), t(get(q + "k.norm")), t(get(q + "o")))
         q = p + "right."
+        r.conv = int(get(q + "conv").shape[1])                 # the taps are what the checkpoint holds
+        if r.conv > sm.CONV_MAX_TAPS:
+            raise ValueError(f"{where}: {r.conv} convolution taps exceed {sm.CONV_MAX_TAPS}")
         hp = torch.stack([-torch.exp(get(q + "A_log").double()), get(q + "dt_bias").double(), get(q + "D").double()])
         right = _Ssd(r, t(get(q + "in")), f(get(q + "conv")), f(get(q + "conv.b")), f(hp), f(get(q + "norm")),
                      t(get(q + "o")))
@@ -429,8 +432,10 @@ class SemanexModel(StreamModel):
                 mixer.right.state = len(self._state_shapes)
                 self._state_shapes.append(((max(r.conv - 1, 0), r.conv_channels), (r.heads, r.state * r.vdim)))
             lay = _Layer(float(get(p + "norm1").float()), mixer, None)
-            if c.canon_taps and self._has(get, p + "canon1"):      # a checkpoint settles optional parts by its tensors
+            if self._has(get, p + "canon1"):      # a checkpoint settles optional parts by its tensors, taps included
                 lay.taps = f(get(p + "canon1"))
+                if lay.taps.shape[1] > sm.CONV_MAX_TAPS:
+                    raise ValueError(f"layer {i}: {lay.taps.shape[1]} convolution taps exceed {sm.CONV_MAX_TAPS}")
                 lay.canon = len(self._state_shapes)
                 self._state_shapes.append(((lay.taps.shape[1] - 1, c.hidden), None))
             if L.ff:

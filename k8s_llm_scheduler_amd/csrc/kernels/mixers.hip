@@ -597,13 +597,15 @@ __global__ __launch_bounds__(64 * NWV) void latent_attention_mfma_kernel(
   }
 }
 
-// out[t][head] = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the key splits
+// out[t][head] = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s over the key splits; workgroups (token, head, slice of
+// the latent columns)
 __global__ void latent_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ pacc,
                                     const float* __restrict__ pml, const int* __restrict__ positions, int C, int H,
                                     int HP, int nsplit, const float* __restrict__ sinks) {
   const int t = blockIdx.x, hd = blockIdx.y;
+  const int d0 = blockIdx.z * blockDim.x + threadIdx.x, dstep = blockDim.x * gridDim.z;
   if (positions[t] < 0) {
-    for (int d = threadIdx.x; d < C; d += blockDim.x) out[((size_t)t * H + hd) * C + d] = 0;
+    for (int d = d0; d < C; d += dstep) out[((size_t)t * H + hd) * C + d] = 0;
     return;
   }
   const size_t rec0 = ((size_t)t * HP + hd) * nsplit;
@@ -614,7 +616,7 @@ __global__ void latent_merge_kernel(bf16_t* __restrict__ out, const float* __res
     const float ms = pml[(rec0 + s) * 2];
     if (ms != -INFINITY) den += expf(ms - M) * pml[(rec0 + s) * 2 + 1];
   }
-  for (int d = threadIdx.x; d < C; d += blockDim.x) {
+  for (int d = d0; d < C; d += dstep) {
     float a = 0.f;
     for (int s = 0; s < nsplit; ++s) {
       const float ms = pml[(rec0 + s) * 2];
@@ -783,7 +785,7 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
   else K8S_LM(32, 20, false);
 #undef K8S_LM
   if (nsplit > 1)
-    latent_merge_kernel<<<dim3(T, H), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16, nsplit,
-                                                   sinks);
+    latent_merge_kernel<<<dim3(T, H, (C + 127) / 128), 128, 0, s>>>((bf16_t*)out, pacc, pml, positions, C, H, HG * 16,
+                                                                    nsplit, sinks);
   return (int)hipGetLastError();
 }

@@ -758,7 +758,8 @@ extern "C" int k8s_latent_attention_mfma(void* out, float* pacc, float* pml, con
   if (!k8s_latent_mfma_ok(C, R, Dn) || H <= 0 || bs <= 0 || nsplit < 1 || (nsplit > 1 && (!pacc || !pml))) return -1;
   const int L = C + R, HG = (H + 15) / 16;
   const size_t lds = (size_t)32 * (L + 8) * 2;
-  const int bt_lds = (size_t)max_blocks * sizeof(int) <= 24576;     // the block table of one sequence beside the key tile
+  // the block table of one sequence beside the key tile, within the 64 KB a launch gets without asking for more
+  const int bt_lds = lds + (size_t)max_blocks * sizeof(int) <= 65536;
   const size_t bt_bytes = bt_lds ? (size_t)max_blocks * sizeof(int) : 0;
   const bool tiles = nsplit == 1 && cu_q != nullptr && nseq > 0 && max_qlen > 1;
   if (tiles && nseq > 65535) return -2;

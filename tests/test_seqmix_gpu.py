@@ -689,3 +689,22 @@ def test_ssd_scan(H, G, N, V):
         o2 = sm.gated_scan(*args(DEV, s2), chunk=chunk, **kw(DEV))
         close(o2, oc, 2e-5)
         close(s2, sc, 1e-4)
+
+
+@pytest.mark.parametrize("width", [64, 5000, 9000])
+def test_latent_attention_prompt_with_long_block_tables(width):
+    """Block tables of many entries per sequence: staged in LDS beside the key tile while they fit, read from memory
+    when they do not; the same rows either way."""
+    torch.manual_seed(56)
+    dt, tol = torch.bfloat16, 2e-2
+    cu, pos, slots, tok_seq = batch()
+    H, Dn, R, C, bs, per = 4, 16, 64, 512, 16, 2
+    cache = torch.randn(4 * per * bs, C + R).to(dt)
+    bt = torch.zeros(4, width, dtype=torch.int32)
+    bt[:, :per] = torch.randperm(4 * per).view(4, per).int()
+    q = torch.randn(T, H * (Dn + R)).to(dt)
+    qabs = (torch.randn(T, H, C) * 0.3).to(dt)
+    oc = sm.latent_attention(qabs, q, cache, bt[:, :per].contiguous(), tok_seq, pos, C, R, H, Dn, 0, 0.2, bs)
+    og = sm.latent_attention(qabs.to(DEV), q.to(DEV), cache.to(DEV), bt.to(DEV), tok_seq.to(DEV), pos.to(DEV), C, R, H, Dn,
+                             0, 0.2, bs, cu_q=cu.to(DEV), max_qlen=27)
+    close(og, oc, tol)
